@@ -25,7 +25,53 @@ inline int32_t f2i(float f) {
 
 EngineCore::EngineCore(const CoreConfig& cfg, std::shared_ptr<const Grammar> grammar)
     : cfg_(cfg), max_batched_tokens0_(cfg.max_batched_tokens), grammar_(std::move(grammar)),
-      bm_(cfg.num_blocks, cfg.block_size) {}
+      bm_(cfg.num_blocks, cfg.block_size) {
+  for (int32_t i = cfg.num_state_slots - 1; i >= 0; --i) free_slots_.push_back(i);  // pop 0,1,...
+}
+
+bool EngineCore::take_slot(Seq& s) {
+  if (cfg_.num_state_slots <= 0 || s.state_slot >= 0) return true;
+  if (free_slots_.empty()) return false;
+  s.state_slot = free_slots_.back();
+  free_slots_.pop_back();
+  s.state_gen = 0;
+  return true;
+}
+
+void EngineCore::drop_slot(Seq& s) {
+  if (s.state_slot >= 0) free_slots_.push_back(s.state_slot);
+  s.state_slot = -1;
+  s.state_gen = 0;
+}
+
+void EngineCore::append(int32_t id, const int32_t* tokens, int32_t n) {
+  if (id < 0 || id >= (int32_t)seqs_.size() || !seqs_[id].live) throw std::runtime_error("append: unknown sequence");
+  Seq& s = seqs_[id];
+  if (!s.p.hold || s.status == S_FINISHED) throw std::runtime_error("append: not a live hold request");
+  if ((int64_t)s.tokens.size() + n > cfg_.max_model_len) throw std::runtime_error("append: past max_model_len");
+  s.tokens.insert(s.tokens.end(), tokens, tokens + n);
+  s.prompt_len = (int32_t)s.tokens.size();
+}
+
+void EngineCore::want(int32_t id, const int32_t* positions, int32_t n) {
+  if (id < 0 || id >= (int32_t)seqs_.size() || !seqs_[id].live) throw std::runtime_error("want: unknown sequence");
+  Seq& s = seqs_[id];
+  for (int32_t i = 0; i < n; ++i) {
+    if (positions[i] < s.num_cached || (!s.want.empty() && positions[i] <= s.want.back()))
+      throw std::runtime_error("want: positions must ascend and lie ahead of the computed tokens");
+    s.want.push_back(positions[i]);
+  }
+}
+
+// Logits rows a scheduled row of q tokens from position p0 produces.
+int32_t EngineCore::logit_rows_of(const Seq& s, int32_t p0, int32_t q, bool section_a) const {
+  if (s.p.hold) {
+    int32_t n = 0;
+    for (size_t i = (size_t)s.want_lo; i < s.want.size() && s.want[i] < p0 + q; ++i) ++n;
+    return n;
+  }
+  return section_a ? 1 : (p0 + q == (int32_t)s.tokens.size());
+}
 
 // ------------------------------------------------------------------ requests
 int32_t EngineCore::add(const int32_t* prompt, int32_t n, const SeqParams& p, double t_arrival) {
@@ -107,7 +153,8 @@ bool EngineCore::grow(Seq& s, int32_t upto) {
 
 void EngineCore::admit(Seq& s) {
   const int32_t bs = cfg_.block_size;
-  if (!cfg_.prefix_cache || s.prompt_len <= bs) return;
+  // a cached page holds no recurrent state, and a hold request's prompt is not final
+  if (!cfg_.prefix_cache || s.prompt_len <= bs || cfg_.num_state_slots > 0 || s.p.hold) return;
   const int32_t nfull = s.prompt_len / bs;
   s.block_hashes.resize(nfull);
   uint64_t h = 0;
@@ -141,6 +188,7 @@ void EngineCore::preempt(int32_t id) {
   s.blocks.clear();
   s.num_cached = 0;
   s.num_registered = 0;
+  drop_slot(s);
   s.status = S_WAITING;
   auto it = std::find(running_.begin(), running_.end(), id);
   if (it != running_.end()) running_.erase(it);
@@ -167,6 +215,7 @@ void EngineCore::finish(int32_t id, FinishReason why, double now, std::vector<in
   s.t_finish = now;
   if (!s.blocks.empty()) bm_.release(s.blocks.data(), (int32_t)s.blocks.size());
   s.blocks.clear();
+  drop_slot(s);
   out.push_back(id);
 }
 
@@ -218,7 +267,9 @@ void EngineCore::schedule(double now) {
     Seq& s = seqs_[id];
     if (s.blocks.empty()) admit(s);
     const int32_t q = std::min(s.pending(), budget);
+    if (cfg_.num_state_slots > 0 && free_slots_.empty() && s.state_slot < 0) break;
     if (!grow(s, s.num_cached + q)) break;
+    take_slot(s);
     waiting_.pop_front();
     s.status = S_RUNNING;
     if (!s.t_first_sched) s.t_first_sched = now;
@@ -303,7 +354,8 @@ int64_t EngineCore::payload_bound() const {
   for (auto& k : graph_keys_) T = std::max<int64_t>(T, k.second);
   const int64_t maxb = (cfg_.max_model_len + cfg_.block_size - 1) / cfg_.block_size;
   const int64_t WA = T * cfg_.group / 16 + N + 1, WB = T / 32 + N + 1;
-  return 2 * N + 3 * T + 2 * N * maxb + 6 * N + 2 * WA + 2 * WB + 3 * N + 64;
+  // + 3 T state rows, + 5 (T - N) logits rows of hold requests (every token may be wanted)
+  return 2 * N + 3 * T + 2 * N * maxb + 6 * N + 2 * WA + 2 * WB + 3 * N + 8 * T + 64;
 }
 
 // --------------------------------------------------------------------- pack
@@ -328,14 +380,16 @@ int64_t EngineCore::schedule_and_pack(int32_t* header, int32_t* payload, int64_t
     maxb = std::max(maxb, (int32_t)seqs_[r.id].blocks.size());
     max_ctx = std::max(max_ctx, seqs_[r.id].num_cached + r.q);
   }
-  int32_t S = (int32_t)A.size();
+  int32_t S = 0;
+  for (auto& r : A) S += logit_rows_of(seqs_[r.id], seqs_[r.id].num_cached, r.q, true);
   for (auto& r : B) {
     TB += r.q;
     WB += (r.q + cfg_.prefill_qblk - 1) / cfg_.prefill_qblk;
     maxb = std::max(maxb, (int32_t)seqs_[r.id].blocks.size());
     const Seq& s = seqs_[r.id];
-    S += (s.num_cached + r.q == (int32_t)s.tokens.size());
+    S += logit_rows_of(s, s.num_cached, r.q, false);
   }
+  const bool stateful = cfg_.num_state_slots > 0;
   const int32_t T = TA + TB, NA = (int32_t)A.size(), NB = (int32_t)B.size();
   int32_t gnb = 0, gtb = 0;
   const bool graph = cfg_.is_cuda && cfg_.use_graphs && NB == 0 && graph_key(NA, T, gnb, gtb);
@@ -350,7 +404,7 @@ int64_t EngineCore::schedule_and_pack(int32_t* header, int32_t* payload, int64_t
     splits = decode_splits(NA, max_ctx, false);
   }
   const int64_t need = 2 * (int64_t)Sh + 3 * (int64_t)Th + (int64_t)NAh * maxb + 3 * NAh + 2 * WAh +
-                       (int64_t)NB * maxb + 3 * NB + 2 * WB + 3 * Sh;
+                       (int64_t)NB * maxb + 3 * NB + 2 * WB + 3 * Sh + (stateful ? 3 * (int64_t)Th : 0);
   if (need > capacity) throw std::runtime_error("step payload exceeds the staging buffer");
 
   int64_t* seeds = reinterpret_cast<int64_t*>(payload);     // payload is 8-byte aligned
@@ -372,6 +426,34 @@ int64_t EngineCore::schedule_and_pack(int32_t* header, int32_t* payload, int64_t
   int32_t* lidx = b_wq + WB;
   int32_t* midx = lidx + Sh;
   int32_t* temps = midx + Sh;
+  // stateful models: per token row, the state slot of its sequence (slot * 2 + the half
+  // to read; -1 = none), its index inside the scheduled run of its sequence, and how many
+  // tokens of that run follow it
+  int32_t* row_state = temps + Sh;
+  int32_t* row_back = row_state + Th;
+  int32_t* row_fwd = row_back + Th;
+  row_pos_.clear();
+  auto state_rows = [&](const Seq& s, int32_t t0, int32_t q) {
+    if (!stateful) return;
+    for (int32_t i = 0; i < q; ++i) {
+      row_state[t0 + i] = s.state_slot < 0 ? -1 : s.state_slot * 2 + (s.state_gen & 1);
+      row_back[t0 + i] = i;
+      row_fwd[t0 + i] = q - 1 - i;
+    }
+  };
+  auto logit_rows = [&](const Seq& s, int32_t id, int32_t t0, int32_t p0, int32_t q, bool a, int32_t& k) {
+    if (s.p.hold) {
+      for (size_t i = (size_t)s.want_lo; i < s.want.size() && s.want[i] < p0 + q; ++i) {
+        lidx[k++] = t0 + (s.want[i] - p0);
+        rows_.push_back({id, false});
+        row_pos_.push_back({id, s.want[i]});
+      }
+    } else if (a || p0 + q == (int32_t)s.tokens.size()) {
+      lidx[k++] = t0 + q - 1;
+      rows_.push_back({id, p0 + q == (int32_t)s.tokens.size()});
+      row_pos_.push_back({id, p0 + q - 1});
+    }
+  };
 
   int32_t t = 0, w = 0, k = 0;
   for (int32_t j = 0; j < NA; ++j) {
@@ -396,9 +478,8 @@ int64_t EngineCore::schedule_and_pack(int32_t* header, int32_t* payload, int64_t
       a_ws[w] = j;
       a_wct[w] = c;
     }
-    lidx[k] = t + r.q - 1;
-    rows_.push_back({r.id, p0 + r.q == (int32_t)s.tokens.size()});
-    ++k;
+    state_rows(s, t, r.q);
+    logit_rows(s, r.id, t, p0, r.q, true, k);
     t += r.q;
   }
   w = 0;
@@ -424,13 +505,12 @@ int64_t EngineCore::schedule_and_pack(int32_t* header, int32_t* payload, int64_t
       b_ws[w] = j;
       b_wq[w] = c;
     }
-    if (p0 + r.q == (int32_t)s.tokens.size()) {
-      lidx[k] = t + r.q - 1;
-      rows_.push_back({r.id, true});
-      ++k;
-    }
+    state_rows(s, t, r.q);
+    logit_rows(s, r.id, t, p0, r.q, false, k);
     t += r.q;
   }
+  int32_t nsamp = 0;
+  for (int32_t i = 0; i < k; ++i) nsamp += rows_[i].second;
   for (int32_t i = 0; i < k; ++i) {
     const Seq& s = seqs_[rows_[i].first];
     midx[i] = s.p.grammar && s.has_gs ? s.mask_idx : -1;
@@ -439,6 +519,8 @@ int64_t EngineCore::schedule_and_pack(int32_t* header, int32_t* payload, int64_t
   }
   if (graph) {   // pad to the captured bucket: padding rows touch only the scratch page
     for (int32_t i = T; i < Th; ++i) { ids[i] = 0; pos[i] = 0; slots[i] = -1; }
+    if (stateful)
+      for (int32_t i = T; i < Th; ++i) { row_state[i] = -1; row_back[i] = 0; row_fwd[i] = 0; }
     for (int32_t j = NA; j < NAh; ++j) {
       std::fill(a_bt + (int64_t)j * maxb, a_bt + (int64_t)(j + 1) * maxb, cfg_.scratch_block);
       a_qs[j] = 0; a_ql[j] = 0; a_kvl[j] = 1;
@@ -451,6 +533,9 @@ int64_t EngineCore::schedule_and_pack(int32_t* header, int32_t* payload, int64_t
   header[H_T] = Th; header[H_TA] = TAh; header[H_NA] = NAh; header[H_WA] = WAh;
   header[H_NB] = NB; header[H_WB] = WB; header[H_S] = Sh; header[H_MAXB] = maxb;
   header[H_SPLITS] = splits; header[H_PAYLOAD] = (int32_t)need; header[H_TILES] = NTL;
+  header[H_STATE] = stateful ? 1 : 0;
+  // rows that sample; a graph replays its sampler whatever the rows are
+  header[H_NSAMP] = graph ? Sh : nsamp;
   ++num_steps;
   return need;
 }
@@ -459,10 +544,15 @@ int64_t EngineCore::schedule_and_pack(int32_t* header, int32_t* payload, int64_t
 std::vector<int32_t> EngineCore::post(const int32_t* sampled, int32_t n, double now) {
   std::vector<int32_t> done;
   done.swap(finished_);
-  for (int32_t id : decode_) seqs_[id].num_cached += 1;
+  for (int32_t id : decode_) {
+    seqs_[id].num_cached += 1;
+    seqs_[id].state_gen += 1;
+  }
   for (auto& r : extend_) {
     Seq& s = seqs_[r.id];
     s.num_cached += r.q;
+    s.state_gen += 1;
+    while (s.want_lo < (int32_t)s.want.size() && s.want[s.want_lo] < s.num_cached) ++s.want_lo;
     publish(s);
     if (!s.t_prefill_done && !s.in_prefill()) s.t_prefill_done = now;
   }

@@ -44,6 +44,10 @@ struct SeqParams {
   bool grammar = true;
   int32_t min_items = 0;
   int32_t profile = 0;                   // grammar profile (grammar.h Profile)
+  // scoring request: nothing is sampled or appended; its tokens arrive with add() and
+  // append(), logits are produced for the positions given to want(), and it stays live
+  // (keeping its pages and state slot between steps) until abort() retires it
+  bool hold = false;
 };
 
 struct Seq {
@@ -60,6 +64,14 @@ struct Seq {
   State gs{};
   int32_t mask_idx = -1;
   int32_t num_sampled = 0, num_forced = 0;
+  // per-sequence recurrent state (models that carry one besides the paged KV): the slot
+  // in the device state pool, and how many steps have advanced it.  The pool is double
+  // buffered: a step reads half (state_gen & 1) and writes the other one, so rows of one
+  // launch never read what other rows of the same launch write.
+  int32_t state_slot = -1;
+  int32_t state_gen = 0;
+  std::vector<int32_t> want;             // hold: positions whose logits are asked for (ascending)
+  int32_t want_lo = 0;                   // first entry of want not yet produced
   SeqStatus status = S_WAITING;
   FinishReason finish = F_NONE;
   double t_arrival = 0, t_first_sched = 0, t_prefill_done = 0, t_first_token = 0, t_finish = 0;
@@ -81,6 +93,7 @@ struct CoreConfig {
   int32_t hkv = 8;                       // local kv heads (decode split heuristic)
   int32_t decode_tiles = 1;              // 16-column tiles per decode attention work item
   int32_t prefill_qblk = 32;             // queries per prefill attention work item (32 | 64)
+  int32_t num_state_slots = 0;           // > 0: every running sequence owns a state slot
   bool jump_forward = true;
   bool prefix_cache = true;
   bool is_cuda = true;
@@ -92,7 +105,7 @@ struct CoreConfig {
 // header slots (must match runner.py)
 enum : int {
   H_T = 0, H_TA, H_NA, H_WA, H_NB, H_WB, H_S, H_MAXB, H_GNB, H_GTB, H_SPLITS, H_PAYLOAD, H_STOP,
-  H_TILES, HEADER = 16
+  H_TILES, H_STATE, H_NSAMP, HEADER = 16
 };
 
 class EngineCore {
@@ -101,6 +114,12 @@ class EngineCore {
 
   // --- requests
   int32_t add(const int32_t* prompt, int32_t n, const SeqParams& p, double t_arrival);
+  // More tokens for a hold request (a prompt that arrives in portions): they are
+  // pending from the next step on.
+  void append(int32_t id, const int32_t* tokens, int32_t n);
+  // Positions (absolute, ascending over all calls) of a hold request whose logits the
+  // steps that run them must produce.
+  void want(int32_t id, const int32_t* positions, int32_t n);
   void release(int32_t id);              // forget a finished sequence's record
   std::vector<int32_t> abort_all(FinishReason why, double now);
   // Retire one queued/running sequence between steps (releases its blocks).
@@ -138,6 +157,9 @@ class EngineCore {
   // of blocks pinned.
   int32_t pin_prefix(const int32_t* tokens, int32_t n);
   int32_t num_pinned() const { return (int32_t)pinned_.size(); }
+  int32_t num_free_state_slots() const { return (int32_t)free_slots_.size(); }
+  // (sequence id, position) of every logits row of the last packed step, in row order
+  const std::vector<std::pair<int32_t, int32_t>>& logit_rows() const { return row_pos_; }
 
   // --- inspection
   const Seq& seq(int32_t id) const { return seqs_[id]; }
@@ -156,6 +178,9 @@ class EngineCore {
   void admit(Seq& s);
   void publish(Seq& s);
   void preempt(int32_t id);
+  bool take_slot(Seq& s);
+  void drop_slot(Seq& s);
+  int32_t logit_rows_of(const Seq& s, int32_t p0, int32_t q, bool section_a) const;
   int32_t preempt_victim(int32_t exclude) const;
   void finish(int32_t id, FinishReason why, double now, std::vector<int32_t>& out);
   void schedule(double now);
@@ -179,6 +204,8 @@ class EngineCore {
   std::vector<int32_t> scratch_;
   std::vector<int32_t> finished_;
   std::vector<int32_t> pinned_;
+  std::vector<int32_t> free_slots_;
+  std::vector<std::pair<int32_t, int32_t>> row_pos_;
 };
 
 }  // namespace rfqrt

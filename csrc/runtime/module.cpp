@@ -185,6 +185,7 @@ PYBIND11_MODULE(_runtime, m) {
              geti("hkv", cfg.hkv);
              geti("decode_tiles", cfg.decode_tiles);
              geti("prefill_qblk", cfg.prefill_qblk);
+             geti("num_state_slots", cfg.num_state_slots);
              if (cfg.prefill_qblk != 32 && cfg.prefill_qblk != 64)
                throw py::value_error("prefill_qblk must be 32 or 64");
              getb("jump_forward", cfg.jump_forward);
@@ -198,10 +199,20 @@ PYBIND11_MODULE(_runtime, m) {
            }), py::arg("config"), py::arg("grammar") = nullptr)
       .def("add", [](EngineCore& e, arr<int32_t> prompt, float temperature, int32_t max_tokens,
                      int64_t seed, bool grammar, int32_t min_items, int32_t profile,
-                     double t_arrival) {
-        SeqParams p{temperature, max_tokens, seed, grammar, min_items, profile};
+                     double t_arrival, bool hold) {
+        SeqParams p{temperature, max_tokens, seed, grammar, min_items, profile, hold};
         return e.add(prompt.data(), (int32_t)prompt.size(), p, t_arrival);
+      }, py::arg("prompt"), py::arg("temperature"), py::arg("max_tokens"), py::arg("seed"),
+         py::arg("grammar"), py::arg("min_items"), py::arg("profile"), py::arg("t_arrival"),
+         py::arg("hold") = false)
+      .def("append", [](EngineCore& e, int32_t id, arr<int32_t> tokens) {
+        e.append(id, tokens.data(), (int32_t)tokens.size());
       })
+      .def("want", [](EngineCore& e, int32_t id, arr<int32_t> positions) {
+        e.want(id, positions.data(), (int32_t)positions.size());
+      })
+      .def("logit_rows", [](const EngineCore& e) { return e.logit_rows(); })
+      .def_property_readonly("num_free_state_slots", &EngineCore::num_free_state_slots)
       .def("schedule_and_pack", [](EngineCore& e, py::array_t<int32_t, py::array::c_style> header,
                                    py::array_t<int32_t, py::array::c_style> payload, double now) {
         if (header.size() < HEADER) throw py::value_error("header must hold 16 int32");
@@ -256,6 +267,8 @@ PYBIND11_MODULE(_runtime, m) {
         d["status"] = (int)s.status;
         d["finish"] = (int)s.finish;
         d["mask_idx"] = s.mask_idx;
+        d["state_slot"] = s.state_slot;
+        d["state_gen"] = s.state_gen;
         d["t_first_sched"] = s.t_first_sched;
         d["t_prefill_done"] = s.t_prefill_done;
         d["t_first_token"] = s.t_first_token;

@@ -89,16 +89,49 @@ def _link(out: Path, objs, libs, key_extra: str):
     stamp.write_text(key)
 
 
-def build_kernels(jobs: int | None = None, verbose: bool = False) -> Path:
-    tdir, abi = _torch_paths()
-    headers = sorted((CSRC / "kernels").glob("*.h")) + sorted((CSRC / "comm").glob("*.h"))
-    kernel_srcs = sorted((CSRC / "kernels").glob("*.hip")) + sorted((CSRC / "comm").glob("*.hip"))
-    bind_flags = [
+MIX_SO = PKG_DIR / "_C_mix.so"
+# trap of this hardware generation: some packed-fp32 forms the compiler picks by itself
+# have given wrong results, so the new library is built without them
+MIX_FLAGS = KERNEL_FLAGS + ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _bind_flags(tdir, abi):
+    return [
         "-O2", "-fPIC", "-std=c++17", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-DUSE_ROCM=1",
         "-D__HIP_PLATFORM_AMD__=1", f"-I{tdir / 'include'}",
         f"-I{tdir / 'include' / 'torch' / 'csrc' / 'api' / 'include'}",
         f"-I{sysconfig.get_paths()['include']}", "-Wno-deprecated-declarations",
     ]
+
+
+def build_mix_kernels(verbose: bool = False) -> Path:
+    """``_C_mix.so``: the kernels of the layer-list models (csrc/kernels/mix_*.hip) and
+    their bindings (csrc/bindings/mix_ops.cpp, ``TORCH_LIBRARY(rfq_mix)``) -- a library of
+    its own, so that serving such a model compiles nothing else."""
+    tdir, abi = _torch_paths()
+    headers = sorted((CSRC / "kernels").glob("mix_*.h"))
+    srcs = sorted((CSRC / "kernels").glob("mix_*.hip"))
+    with cf.ThreadPoolExecutor(min(8, len(srcs) + 1)) as ex:
+        futs = [ex.submit(_compile, s, MIX_FLAGS + [f"-I{CSRC / 'kernels'}"], headers, "m")
+                for s in srcs]
+        futs.append(ex.submit(_compile, CSRC / "bindings" / "mix_ops.cpp", _bind_flags(tdir, abi),
+                              headers, "mb"))
+        objs = [f.result() for f in futs]
+    libs = [f"-L{tdir / 'lib'}", "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
+            f"-Wl,-rpath,{tdir / 'lib'}"]
+    _link(MIX_SO, objs, libs, "M" + ARCH)
+    _check_stubs(MIX_SO)
+    if verbose:
+        print(f"[rfq build] {MIX_SO}")
+    return MIX_SO
+
+
+def build_kernels(jobs: int | None = None, verbose: bool = False) -> Path:
+    tdir, abi = _torch_paths()
+    headers = sorted((CSRC / "kernels").glob("*.h")) + sorted((CSRC / "comm").glob("*.h"))
+    kernel_srcs = sorted(s for s in (CSRC / "kernels").glob("*.hip") if not s.name.startswith("mix_")) \
+        + sorted((CSRC / "comm").glob("*.hip"))
+    bind_flags = _bind_flags(tdir, abi)
     jobs = jobs or min(8, os.cpu_count() or 4)
     with cf.ThreadPoolExecutor(jobs) as ex:
         futs = [ex.submit(_compile, s, KERNEL_FLAGS + [f"-I{CSRC / 'kernels'}"], headers, "k")
@@ -161,6 +194,7 @@ def build_runtime(verbose: bool = False) -> Path:
 def build_all(verbose: bool = True) -> None:
     build_runtime(verbose)
     build_kernels(verbose=verbose)
+    build_mix_kernels(verbose=verbose)
 
 
 if __name__ == "__main__":

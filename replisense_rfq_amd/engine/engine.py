@@ -28,14 +28,14 @@ import numpy as np
 import torch
 
 from .. import runtime
-from ..models.config import get_config
+from ..models.config import LayeredConfig, get_config, load_config
 from ..models.llama import DecoderLM
 from ..parallel.tp import SINGLE, TPContext
 from ..utils.config import EngineConfig
 from ..utils.faults import CustomAllReduceError, FaultInjector
 from ..utils.trace import trace_range
 from .grammar import PROFILE_REFERENCE, PROFILE_SYNTHETIC, get_grammar
-from .kv_cache import KVCache
+from .kv_cache import KVCache, LayeredKVCache
 from .runner import EXT_MAX, MAX_GRAPH_TOKENS, TOKEN_MULTS, ModelRunner
 from .sequence import SamplingParams, Sequence, Status
 from .tokenizer import flavor_for_vocab, get_tokenizer
@@ -80,16 +80,32 @@ class LLMEngine:
             torch.cuda.set_device(self.device)
         if tp.enabled and self.cfg.custom_allreduce and self.device.type == "cuda":
             tp.enable_custom_allreduce()
-        self.model_cfg = get_config(self.cfg.model)
-        self.tokenizer = get_tokenizer(flavor_for_vocab(self.model_cfg.vocab_size),
-                                       self._tokenizer_path())
+        # a checkpoint folder whose config.json names a known architecture decides the
+        # model class; otherwise the configuration is one of the named ones
+        self.model_cfg = (model.cfg if model is not None else None) \
+            or (load_config(self.cfg.weights_path) if self.cfg.weights_path else None) \
+            or get_config(self.cfg.model)
+        self.layered = isinstance(self.model_cfg, LayeredConfig)
+        self.dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[self.cfg.dtype]
+        if self.dtype != torch.bfloat16 and not self.layered:
+            raise ValueError("the Llama / Mixtral kernels are bf16 only")
+        self.tokenizer = self._make_tokenizer()
         t0 = time.perf_counter()
         weights = None
         if model is None and self.cfg.weights_path:
-            from ..models.weights import load_safetensors
+            from ..models.weights import load_layered_safetensors, load_safetensors
 
-            weights = load_safetensors(self.cfg.weights_path, self.model_cfg, tp, self.device,
-                                       moe_ep=self.cfg.moe_parallel == "ep")
+            if self.layered:
+                weights = load_layered_safetensors(self.cfg.weights_path, self.model_cfg,
+                                                   self.device, self.dtype)
+            else:
+                weights = load_safetensors(self.cfg.weights_path, self.model_cfg, tp, self.device,
+                                           moe_ep=self.cfg.moe_parallel == "ep")
+        if model is None and self.layered:
+            from ..models.livisun import LivisunLM
+
+            model = LivisunLM(self.model_cfg, self.device, tp, seed=self.cfg.seed,
+                              weights=weights, dtype=self.dtype)
         self.model = model or DecoderLM(self.model_cfg, self.device, tp, seed=self.cfg.seed,
                                         weights=weights, moe_ep=self.cfg.moe_parallel == "ep")
         # the norm weights go into qkv / gate|up before anything copies those weights
@@ -99,11 +115,17 @@ class LLMEngine:
         # before the KV pool is sized from the free memory: the tiled copies take theirs
         self.tiled_bytes = self.model.tile_decode_weights() if self.cfg.tune_gemm else 0
         self.init_weights_s = time.perf_counter() - t0
-        self.kv = KVCache(self.model_cfg, self.model.hkv, self._num_blocks(), self.device,
-                          prefix_cache=self.cfg.prefix_cache)
-        self.model.attach_kv_cache(self.kv.k, self.kv.v)
-        self.grammar = get_grammar(self.tokenizer.flavor, self.tokenizer) if self.cfg.grammar \
-            else None
+        if self.layered:
+            # one state slot per sequence in flight; slot and pages are handed out together
+            self.kv = LayeredKVCache(self.model_cfg, self._num_blocks(), self.device,
+                                     num_slots=self.cfg.max_num_seqs, dtype=self.dtype)
+            self.model.attach_kv_cache(self.kv.k, self.kv.v, self.kv.state)
+        else:
+            self.kv = KVCache(self.model_cfg, self.model.hkv, self._num_blocks(), self.device,
+                              prefix_cache=self.cfg.prefix_cache)
+            self.model.attach_kv_cache(self.kv.k, self.kv.v)
+        self.grammar = get_grammar(self.tokenizer.flavor, self.tokenizer) \
+            if self.cfg.grammar and self.tokenizer.flavor != "ids" else None
         self.runner = ModelRunner(self.model, self.kv, self.cfg,
                                   self.grammar.mask_table() if self.grammar else None, tp)
         self.core = self._make_core()
@@ -111,7 +133,7 @@ class LLMEngine:
         self._live: dict[int, Sequence] = {}
         self.capture_s = 0.0
         self.tune_s = 0.0
-        if self.device.type == "cuda" and self.cfg.tune_gemm:
+        if self.device.type == "cuda" and self.cfg.tune_gemm and not self.layered:
             self._tune_gemms()
         if capture and self.device.type == "cuda" and self.cfg.use_graphs:
             buckets = [b for b in self.cfg.graph_buckets if b <= self.cfg.max_num_seqs]
@@ -132,7 +154,7 @@ class LLMEngine:
         self.timers = {"execute_s": 0.0, "post_s": 0.0}
         self.faults = FaultInjector()
         self.pinned_blocks = 0
-        if self.cfg.prefix_cache and self.cfg.warm_prefix and tp.rank == 0:
+        if self.cfg.prefix_cache and self.cfg.warm_prefix and tp.rank == 0 and not self.layered:
             try:
                 self.warm_prefix()
             except BaseException:
@@ -159,6 +181,13 @@ class LLMEngine:
         return self.pinned_blocks
 
     # ------------------------------------------------------------------ setup
+    def _make_tokenizer(self):
+        if self.layered and not self._tokenizer_path():
+            from .tokenizer import IdTokenizer
+
+            return IdTokenizer(self.model_cfg.vocab_size, tuple(self.model_cfg.eos_ids))
+        return get_tokenizer(flavor_for_vocab(self.model_cfg.vocab_size), self._tokenizer_path())
+
     def _tokenizer_path(self) -> str | None:
         if self.cfg.tokenizer_path:
             return self.cfg.tokenizer_path
@@ -175,7 +204,8 @@ class LLMEngine:
                     scratch_block=self.kv.scratch_block, max_num_seqs=c.max_num_seqs,
                     max_batched_tokens=c.max_batched_tokens, max_model_len=c.max_model_len,
                     ext_max=EXT_MAX, group=self.model.hq // self.model.hkv, hkv=self.model.hkv,
-                    jump_forward=c.jump_forward, prefix_cache=c.prefix_cache,
+                    num_state_slots=self.kv.num_slots if self.layered else 0,
+                    jump_forward=c.jump_forward, prefix_cache=c.prefix_cache and not self.layered,
                     is_cuda=self.device.type == "cuda", use_graphs=c.use_graphs,
                     token_mults=list(TOKEN_MULTS), eos_ids=list(self.tokenizer.eos_ids),
                     decode_tiles=c.decode_tiles, prefill_qblk=self.runner.prefill_qblk)
@@ -200,7 +230,11 @@ class LLMEngine:
     def _num_blocks(self) -> int:
         cfg = self.cfg
         per_seq = (cfg.max_model_len + 31) // 32
-        if self.device.type == "cuda":
+        if self.device.type == "cuda" and self.layered:
+            free, _ = torch.cuda.mem_get_info(self.device)
+            per = LayeredKVCache.bytes_per_block(self.model_cfg, 32, 2 if self.dtype == torch.bfloat16 else 4)
+            n = max(16, int(free * cfg.kv_fraction) // per)
+        elif self.device.type == "cuda":
             free, _ = torch.cuda.mem_get_info(self.device)
             n = KVCache.blocks_for_memory(self.model_cfg, self.model.hkv, free, cfg.kv_fraction)
         else:
@@ -225,9 +259,43 @@ class LLMEngine:
         seq.core_id = self.core.add(np.asarray(prompt_ids, np.int32), float(params.temperature),
                                     int(params.max_tokens), int(params.seed),
                                     bool(params.grammar and self.grammar is not None),
-                                    int(params.min_items), int(params.profile), seq.t_arrival)
+                                    int(params.min_items), int(params.profile), seq.t_arrival,
+                                    bool(params.hold))
         self._live[seq.core_id] = seq
         return seq
+
+    # ---------------------------------------------------------------- scoring
+    def score_request(self, tokens: list[int], want: list[int] | None = None) -> Sequence:
+        """Admit a scoring request: its tokens are run through the model (nothing is sampled),
+        more tokens may follow with :meth:`score_extend`, and each step returns the logits of
+        the wanted positions.  It keeps its pages and state slot until :meth:`abort_request`."""
+        seq = self.add_request(list(tokens), SamplingParams(temperature=0.0, max_tokens=1,
+                                                            grammar=False, hold=True))
+        if want:
+            self.core.want(seq.core_id, np.asarray(want, np.int32))
+        return seq
+
+    def score_extend(self, seq: Sequence, tokens: list[int], want: list[int] | None = None) -> None:
+        """More tokens for a scoring request; ``want`` holds absolute positions."""
+        self.core.append(seq.core_id, np.asarray(tokens, np.int32))
+        seq.tokens.extend(tokens)
+        if want:
+            self.core.want(seq.core_id, np.asarray(want, np.int32))
+
+    def score_step(self):
+        """One engine step that keeps its logits: returns (rows, logits) with rows =
+        [(Sequence, position)] in the order of the logits' rows, or None if nothing ran."""
+        self.runner.keep_logits = True
+        try:
+            live = dict(self._live)
+            self.step()
+            if self.runner.last_logits is None:
+                return None
+            rows = [(live[i], p) for i, p in self.runner.last_rows]
+            return rows, self.runner.last_logits
+        finally:
+            self.runner.keep_logits = False
+            self.runner.last_logits = None
 
     # ------------------------------------------------------------------- step
     def step(self) -> list[Sequence]:

@@ -46,3 +46,35 @@ class KVCache:
         return {"blocks": self.num_blocks, "free": core.num_free_blocks,
                 "cached": core.num_cached_blocks, "prefix_queries": core.prefix_queries,
                 "prefix_hits": core.prefix_hits, "evictions": core.evictions}
+
+
+class LayeredKVCache:
+    """Pools of a layer-list model: one K and one V pool per layer, each with the layer's
+    own head count and sizes (``[num_blocks, G, block, dim]`` / ``[..., vdim]``), all
+    indexed by the same block ids, plus the state pool of the input convolutions:
+    ``[L, 2 sublayers, 2 * slots, taps - 1, d]`` fp32.  A sequence owns one slot while it
+    runs (native core); the pool is double buffered, a step reads half ``gen & 1`` of the
+    slot and writes the other, so rows of one launch never read what the launch writes."""
+
+    def __init__(self, cfg, num_blocks: int, device, num_slots: int, block_size: int = 32,
+                 dtype=torch.bfloat16, prefix_cache: bool = False):
+        self.cfg = cfg
+        self.block_size = block_size
+        self.num_blocks = num_blocks
+        self.num_slots = num_slots
+        mk = torch.zeros if torch.device(device).type != "cuda" else torch.empty
+        self.k = [mk((num_blocks, ly.mixer.kv_heads, block_size, ly.mixer.dim), dtype=dtype,
+                     device=device) for ly in cfg.layers]
+        self.v = [mk((num_blocks, ly.mixer.kv_heads, block_size, ly.mixer.vdim), dtype=dtype,
+                     device=device) for ly in cfg.layers]
+        self.state = torch.zeros((cfg.n_layers, 2, 2 * num_slots, max(0, cfg.canon_taps - 1),
+                                  cfg.hidden), dtype=torch.float32, device=device)
+        self.scratch_block = num_blocks - 1
+        self.prefix_cache = False            # a cached page carries no convolution state
+        self.core = None
+
+    @staticmethod
+    def bytes_per_block(cfg, block_size: int = 32, dtype_bytes: int = 2) -> int:
+        return cfg.kv_bytes_per_token(dtype_bytes=dtype_bytes) * block_size
+
+    stats = KVCache.stats

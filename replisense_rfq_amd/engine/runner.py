@@ -35,7 +35,7 @@ from ..utils.faults import CustomAllReduceError
 from .kv_cache import KVCache
 
 (H_T, H_TA, H_NA, H_WA, H_NB, H_WB, H_S, H_MAXB, H_GNB, H_GTB, H_SPLITS, H_PAYLOAD,
- H_STOP, H_TILES) = range(14)
+ H_STOP, H_TILES, H_STATE, H_NSAMP) = range(16)
 HEADER = 16
 SAMPLE_SPLITS = 8
 EXT_MAX = 32                 # extends up to this many tokens use the decode kernel
@@ -51,8 +51,14 @@ def _seed64(req_seed: int, pos: int) -> int:
     return x - (1 << 64) if x >= (1 << 63) else x
 
 
-def _layout(T, NA, WA, NB, WB, S, maxb):
-    """(name, length) of every int32 array in the payload, in order."""
+def _layout(T, NA, WA, NB, WB, S, maxb, state=0):
+    """(name, length) of every int32 array in the payload, in order.  ``state``: the step
+    carries the per-row state arrays of a model with per-sequence state slots."""
+    tail = [("row_state", T), ("row_back", T), ("row_fwd", T)] if state else []
+    return _layout_base(T, NA, WA, NB, WB, S, maxb) + tail
+
+
+def _layout_base(T, NA, WA, NB, WB, S, maxb):
     return [("seeds", 2 * S), ("ids", T), ("pos", T), ("slots", T),
             ("a_bt", NA * maxb), ("a_qs", NA), ("a_ql", NA), ("a_kvl", NA), ("a_ws", WA),
             ("a_wct", WA), ("b_bt", NB * maxb), ("b_qs", NB), ("b_ql", NB), ("b_kvl", NB),
@@ -82,9 +88,15 @@ class ModelRunner:
         self._header = np.zeros(HEADER, np.int32)
         self.decode_tiles = int(getattr(cfg, "decode_tiles", 1))
         # validated on every device (a config the GPU kernels cannot run fails at start-up)
-        qblk = ops.prefill_qblk(model.hq, model.hkv)
+        self.stateful = bool(getattr(model, "stateful", False))
+        qblk = ops.MIXQ_QBLK if self.stateful else ops.prefill_qblk(model.hq, model.hkv)
         self.prefill_qblk = qblk if self.is_cuda else 32
+        # scoring steps (engine.score_step) keep the step's logits and their rows
+        self.keep_logits = False
+        self.last_logits = None
+        self.last_rows = None
         self.ring = None
+        self._core = None
         # SURVEY.md §5.2 debug check: Inf/NaN logits are counted on device inside the step
         # (captured into the decode graphs too) and read back with the sampled tokens
         self.check_finite = bool(getattr(cfg, "check_finite", False))
@@ -92,7 +104,7 @@ class ModelRunner:
         # bounded in-launch waits (stream-K slabs, persistent decode stages) count their
         # timeouts in host-mapped words (csrc/kernels/kerr.hip); allocated here, before
         # any graph capture, and compared after every step's token readback
-        self._kerr0 = ops.kernel_errors()[:2] if self.is_cuda else [0, 0]
+        self._kerr0 = ops.kernel_errors()[:2] if self.is_cuda and not self.stateful else [0, 0]
         if tp.enabled:
             self._setup_control_plane()
         # host-side split of a step: pack (scheduler), launch (upload + forward + sampler
@@ -122,7 +134,7 @@ class ModelRunner:
         T, TA, NA, WA, NB, WB, S, maxb = (int(h[i]) for i in (H_T, H_TA, H_NA, H_WA, H_NB, H_WB,
                                                               H_S, H_MAXB))
         out, o = {}, 0
-        for name, n in _layout(T, NA, WA, NB, WB, S, maxb):
+        for name, n in _layout(T, NA, WA, NB, WB, S, maxb, int(h[H_STATE])):
             out[name] = buf[o:o + n]
             o += n
         out["a_bt"] = out["a_bt"].view(NA, maxb)
@@ -141,7 +153,8 @@ class ModelRunner:
             num_prefill_tokens=T - TA, pf_block_tables=v["b_bt"], pf_q_start=v["b_qs"],
             pf_q_len=v["b_ql"], pf_kv_len=v["b_kvl"], work_seq=v["b_ws"], work_qblk=v["b_wq"],
             logits_idx=v["lidx"], decode_splits=int(h[H_SPLITS]),
-            decode_tiles=max(1, int(h[H_TILES])), prefill_qblk=self.prefill_qblk)
+            decode_tiles=max(1, int(h[H_TILES])), prefill_qblk=self.prefill_qblk,
+            extra={k: v[k] for k in ("row_state", "row_back", "row_fwd") if k in v})
 
     def _staging(self, words: int) -> np.ndarray:
         if self._stage is None or self._stage.size < words:
@@ -177,6 +190,7 @@ class ModelRunner:
         the pinned staging buffer; run it and return the sampled id per logits row
         (None when there is nothing to run)."""
         t0 = time.perf_counter()
+        self._core = core
         buf = self._staging(core.payload_bound())
         n = core.schedule_and_pack(self._header, buf, now)
         self.stats["pack_s"] += time.perf_counter() - t0
@@ -278,7 +292,14 @@ class ModelRunner:
             buf = self._upload(payload)
             v = self._views(buf, header)
             logits = self.model.forward(self._meta(v, header))
-            out = self._sample(logits, v["midx"], v["temps"], v["seeds"])
+            if self.keep_logits:
+                self.last_logits = logits
+                self.last_rows = list(self._core.logit_rows()) if self._core is not None else None
+            if int(header[H_NSAMP]) == 0:
+                # no row of the step samples (prefill chunks that end no prompt, scoring)
+                out = torch.zeros(logits.shape[0], dtype=torch.int32, device=logits.device)
+            else:
+                out = self._sample(logits, v["midx"], v["temps"], v["seeds"])
         t1 = time.perf_counter()
         hook_err = None
         if self.busy_hook is not None:
@@ -307,7 +328,7 @@ class ModelRunner:
                 self._nonfinite.zero_()
                 raise RuntimeError(f"non-finite logits: {bad} Inf/NaN entries in step "
                                    f"{self.stats['steps']} (TP rank {self.tp.rank})")
-        if self.is_cuda:
+        if self.is_cuda and not self.stateful:
             kerr = ops.kernel_errors()
             if kerr[:2] != self._kerr0:
                 # a hand-off inside a launch gave up after its bounded wait: this step's
@@ -379,7 +400,8 @@ class ModelRunner:
             header[[H_T, H_TA, H_NA, H_WA, H_NB, H_WB, H_S, H_MAXB, H_SPLITS]] = \
                 [tb, tb, nb, tb, 0, 0, nb, maxb, self._decode_splits(nb, 0, graph=True)]
             header[H_TILES] = self.decode_tiles
-            n = sum(k for _, k in _layout(tb, nb, tb, 0, 0, nb, maxb))
+            header[H_STATE] = int(self.stateful)
+            n = sum(k for _, k in _layout(tb, nb, tb, 0, 0, nb, maxb, int(self.stateful)))
             gbuf = torch.zeros(n, dtype=torch.int32, device=self.device)
             v = self._views(gbuf, header)
             # a harmless padding state for the capture run: no sequences, no KV writes
@@ -388,6 +410,8 @@ class ModelRunner:
             v["a_kvl"].fill_(1)
             v["midx"].fill_(-1)
             v["a_bt"].fill_(self.kv.scratch_block)
+            if self.stateful:
+                v["row_state"].fill_(-1)
             meta = self._meta(v, header)
             out = torch.zeros(nb, dtype=torch.int32, device=self.device)
 

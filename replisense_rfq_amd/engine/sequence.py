@@ -24,6 +24,7 @@ class SamplingParams:
     min_items: int = 0      # bench-only schema hint: minimum line_items the output must contain
     profile: int = 0        # grammar profile: 0 reference (service default), 1 synthetic
                             # (bench-only caps for random-init weights; grammar/compiler.py)
+    hold: bool = False      # scoring request: runs the tokens it is given, samples nothing
 
 
 @dataclass

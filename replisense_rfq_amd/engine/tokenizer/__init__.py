@@ -159,3 +159,29 @@ def get_tokenizer(flavor: str = "llama3", path: str | None = None) -> Tokenizer:
 
 def flavor_for_vocab(vocab_size: int) -> str:
     return "mixtral" if vocab_size == 32000 else "llama3"
+
+
+class IdTokenizer:
+    """Tokenizer of a model that ships no vocabulary: text is the token ids themselves,
+    written as decimal numbers with blanks between them."""
+    flavor = "ids"
+
+    def __init__(self, vocab_size: int, eos_ids: tuple = ()):
+        self.vocab_size = vocab_size
+        self.eos_ids = tuple(eos_ids)
+        self.bos_id = None
+
+    def encode(self, text: str) -> list[int]:
+        ids = [int(t) for t in text.split()]
+        if any(i < 0 or i >= self.vocab_size for i in ids):
+            raise ValueError("token id outside the vocabulary")
+        return ids
+
+    def encode_batch(self, texts: list[str]) -> list[list[int]]:
+        return [self.encode(t) for t in texts]
+
+    def decode(self, ids, skip_special: bool = True) -> str:
+        return " ".join(str(int(i)) for i in ids)
+
+    def chat_ids(self, messages: list[dict], add_generation_prompt: bool = True) -> list[int]:
+        return [i for m in messages for i in self.encode(m["content"])]

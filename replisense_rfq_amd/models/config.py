@@ -80,3 +80,136 @@ def get_config(name: str) -> ModelConfig:
     if name not in CONFIGS:
         raise KeyError(f"unknown model {name!r}; known: {sorted(CONFIGS)}")
     return CONFIGS[name]
+
+
+# --------------------------------------------------------------------------
+# Layer-list models: config.json names an architecture and lists the layers, each
+# with its own mixer and feed-forward sizes (nothing is shared between layers, so
+# every layer owns its KV pool shape).  Livisun is the first of them.
+@dataclass(frozen=True)
+class MixerSpec:
+    """Attention mixer: H query heads over G key/value heads, per-head query/key
+    size ``dim`` and value size ``vdim``; scores are scaled by ``scale``; position
+    i sees j <= i inside its own block of ``chunk`` positions (0 = plain causal)."""
+    kind: str = "attention"
+    heads: int = 4
+    kv_heads: int = 2
+    dim: int = 64
+    vdim: int = 64
+    scale: float = 0.125
+    chunk: int = 0
+
+    @property
+    def group(self) -> int:
+        return self.heads // self.kv_heads
+
+
+@dataclass(frozen=True)
+class MlpSpec:
+    kind: str = "dense"
+    ff: int = 256
+    limit: float = 7.0
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    mixer: MixerSpec
+    mlp: MlpSpec | None
+
+
+@dataclass(frozen=True)
+class LayeredConfig:
+    name: str
+    architecture: str = "Livisun"
+    vocab_size: int = 512
+    hidden: int = 256
+    layers: tuple = ()
+    rms_eps: float = 1e-5
+    embed_scale: float = 1.0
+    canon_taps: int = 3
+    max_position: int = 8192
+    init_std: float = 0.02
+    bos_id: int = 0
+    eos_ids: tuple = ()
+    n_experts: int = 0
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return False
+
+    def params(self) -> int:
+        d, n = self.hidden, 0
+        for ly in self.layers:
+            m = ly.mixer
+            n += d * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + m.heads * m.vdim * d
+            n += 2 * m.dim + m.heads * m.heads + m.heads + 6 * d + 2 * d * self.canon_taps
+            if ly.mlp is not None:
+                n += 3 * d * ly.mlp.ff
+        return n + 2 * self.vocab_size * d + d
+
+    def kv_bytes_per_token(self, tp: int = 1, dtype_bytes: int = 2) -> int:
+        return sum(ly.mixer.kv_heads * (ly.mixer.dim + ly.mixer.vdim) for ly in self.layers) \
+            * dtype_bytes
+
+    def to_dict(self):
+        return asdict(self)
+
+    @classmethod
+    def from_json(cls, d: dict, name: str | None = None) -> "LayeredConfig":
+        """config.json of a layer-list model: vocab, width, norm.eps, embedding.scale,
+        canon.taps and ``layers`` (type, mixer sizes, mlp or null)."""
+        layers = []
+        for i, ly in enumerate(d["layers"]):
+            if ly["type"] != "attention":
+                raise ValueError(f"layer {i}: unknown mixer type {ly['type']!r}")
+            m = ly["mixer"]
+            if m["heads"] % m["kv_heads"]:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+            mixer = MixerSpec("attention", int(m["heads"]), int(m["kv_heads"]), int(m["dim"]),
+                              int(m["vdim"]), float(m["scale"]),
+                              int((m.get("mask") or {}).get("size", 0)))
+            f = ly.get("mlp")
+            if f is not None and f["kind"] != "dense":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+            mlp = None if f is None else MlpSpec("dense", int(f["ff"]), float(f["limit"]))
+            layers.append(LayerSpec(mixer, mlp))
+        return cls(name=name or d["architecture"].lower(), architecture=d["architecture"],
+                   vocab_size=int(d["vocab"]), hidden=int(d["width"]), layers=tuple(layers),
+                   rms_eps=float(d["norm"]["eps"]), embed_scale=float(d["embedding"]["scale"]),
+                   canon_taps=int(d["canon"]["taps"]),
+                   max_position=int(d.get("max_position", 8192)))
+
+
+def _livisun_layers(n, heads, kv_heads, dim, vdim, chunk, ff, scale=None, limit=7.0):
+    m = MixerSpec("attention", heads, kv_heads, dim, vdim, scale or dim ** -0.5, chunk)
+    return tuple(LayerSpec(m, MlpSpec("dense", ff, limit)) for _ in range(n))
+
+
+# test / smoke size, and layer shapes of the 8B-class comparison in bench.py --arch
+TINY_LIVISUN = LayeredConfig("tiny-livisun", vocab_size=384, hidden=128, embed_scale=4.0,
+                             layers=_livisun_layers(2, 6, 3, 32, 16, 24, 192, limit=1.5))
+LIVISUN_8B = LayeredConfig("livisun-8b", vocab_size=128256, hidden=4096, embed_scale=1.0,
+                           layers=_livisun_layers(32, 32, 8, 128, 128, 2048, 14336))
+CONFIGS.update({c.name: c for c in (TINY_LIVISUN, LIVISUN_8B)})
+
+# config.json "architecture" -> reader
+ARCHITECTURES = {"Livisun": LayeredConfig.from_json}
+
+
+def load_config(path: str):
+    """Model configuration from a checkpoint folder's config.json, chosen by its
+    ``architecture`` key; None when the folder names no architecture known here."""
+    import json
+    import os
+
+    f = os.path.join(path, "config.json") if os.path.isdir(path) else ""
+    if not f or not os.path.exists(f):
+        return None
+    with open(f) as fh:
+        d = json.load(fh)
+    reader = ARCHITECTURES.get(d.get("architecture", ""))
+    return reader(d) if reader else None

@@ -250,3 +250,105 @@ def export_hf(full: dict, cfg: ModelConfig) -> dict[str, torch.Tensor]:
             out[p + "mlp.up_proj.weight"] = lw["gate_up"][F:]
             out[p + "mlp.down_proj.weight"] = lw["down"]
     return {k: v.contiguous() for k, v in out.items()}
+
+
+# --------------------------------------------------------------------------
+# Layer-list models (LayeredConfig).  Tensor names are the checkpoint's own:
+#   embed, head [V, d]; final.norm [d]
+#   l<i>.norm1 | norm1b | norm2 | norm2b | ls1 | ls2 [d]; l<i>.canon1 | canon2 [d, taps]
+#   l<i>.mix.q [H*dim, d]  .k [G*dim, d]  .v [G*vdim, d]  .o [d, H*vdim]
+#   l<i>.mix.q.norm | k.norm [dim]; l<i>.mix.talk [H, H]; l<i>.mix.sink [H]
+#   l<i>.mlp.gate | up [F, d]; l<i>.mlp.down [d, F]
+# Loaded layout per layer: qkv = q|k|v rows and gate_up = gate|up rows in the model's
+# dtype; norm weights, layer scales, convolution taps, talk and sink in fp32.
+LAYERED_F32 = ("norm1", "norm1b", "norm2", "norm2b", "ls1", "ls2", "canon1", "canon2")
+
+
+def _assemble_layer(get, ly, has, dtype, device):
+    lw = LayerWeights()
+    for k in LAYERED_F32:
+        if has(k):
+            lw[k] = get(k).float().contiguous().to(device)
+    lw["qkv"] = torch.cat([get("mix.q"), get("mix.k"), get("mix.v")], 0).to(dtype).contiguous().to(device)
+    lw["o"] = get("mix.o").to(dtype).contiguous().to(device)
+    lw["q_norm"] = get("mix.q.norm").float().to(device)
+    lw["k_norm"] = get("mix.k.norm").float().to(device)
+    lw["talk"] = get("mix.talk").float().contiguous().to(device)
+    lw["sink"] = get("mix.sink").float().to(device)
+    if ly.mlp is not None:
+        lw["gate_up"] = torch.cat([get("mlp.gate"), get("mlp.up")], 0).to(dtype).contiguous().to(device)
+        lw["down"] = get("mlp.down").to(dtype).contiguous().to(device)
+    m = ly.mixer
+    shapes = {"qkv": (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim),), "talk": (m.heads, m.heads),
+              "sink": (m.heads,), "q_norm": (m.dim,), "k_norm": (m.dim,)}
+    for k, shp in shapes.items():
+        if tuple(lw[k].shape[:len(shp)]) != shp:
+            raise ValueError(f"tensor {k}: shape {tuple(lw[k].shape)} does not fit the configuration")
+    return lw
+
+
+def load_layered_safetensors(path: str, cfg, device, dtype=torch.bfloat16) -> dict:
+    import glob
+    import os
+
+    files = sorted(glob.glob(os.path.join(path, "*.safetensors"))) if os.path.isdir(path) else [path]
+    ck = _LazyCheckpoint(files)
+    w = {"embed": ck.full("embed").to(dtype).to(device), "lm_head": ck.full("head").to(dtype).to(device),
+         "final_norm": ck.full("final.norm").float().to(device), "vocab_start": 0, "layers": []}
+    for i, ly in enumerate(cfg.layers):
+        pre = f"l{i}."
+        w["layers"].append(_assemble_layer(lambda k: ck.full(pre + k), ly, lambda k: pre + k in ck,
+                                           dtype, device))
+    return w
+
+
+def init_layered_weights(cfg, device, dtype=torch.bfloat16, seed: int = 0) -> dict:
+    """Seeded random weights of a layer-list model (tests and benchmarks): projections
+    N(0, init_std) scaled so that activations stay O(1), norm weights near one, layer
+    scales, taps, sinks and the head-mixing matrix away from their neutral values so
+    that each of them shows in the logits."""
+    d = cfg.hidden
+    full = {}
+
+    def rnd(name, shape, std, mean=0.0):
+        t = _randn(shape, std, (seed, name), "cpu", torch.float32) + mean
+        full[name] = t.to(torch.bfloat16).float()      # checkpoint precision
+        return full[name]
+
+    rnd("embed", (cfg.vocab_size, d), 1.0)
+    rnd("head", (cfg.vocab_size, d), d ** -0.5)
+    rnd("final.norm", (d,), 0.1, 1.0)
+    for i, ly in enumerate(cfg.layers):
+        m, p = ly.mixer, f"l{i}."
+        for k in ("norm1", "norm1b", "norm2", "norm2b"):
+            rnd(p + k, (d,), 0.1, 1.0)
+        rnd(p + "ls1", (d,), 0.1, 0.5)
+        rnd(p + "ls2", (d,), 0.1, 0.5)
+        rnd(p + "canon1", (d, cfg.canon_taps), 0.3)
+        rnd(p + "canon2", (d, cfg.canon_taps), 0.3)
+        rnd(p + "mix.q", (m.heads * m.dim, d), d ** -0.5)
+        rnd(p + "mix.k", (m.kv_heads * m.dim, d), d ** -0.5)
+        rnd(p + "mix.v", (m.kv_heads * m.vdim, d), d ** -0.5)
+        rnd(p + "mix.o", (d, m.heads * m.vdim), (m.heads * m.vdim) ** -0.5)
+        rnd(p + "mix.q.norm", (m.dim,), 0.1, 1.0)
+        rnd(p + "mix.k.norm", (m.dim,), 0.1, 1.0)
+        full[p + "mix.talk"] = (torch.eye(m.heads) + rnd(p + "mix.talk", (m.heads, m.heads), 0.2)
+                                ).to(torch.bfloat16).float()
+        rnd(p + "mix.sink", (m.heads,), 1.0)
+        if ly.mlp is not None:
+            rnd(p + "mlp.gate", (ly.mlp.ff, d), d ** -0.5)
+            rnd(p + "mlp.up", (ly.mlp.ff, d), d ** -0.5)
+            rnd(p + "mlp.down", (d, ly.mlp.ff), ly.mlp.ff ** -0.5)
+    return layered_from_full(full, cfg, device, dtype)
+
+
+def layered_from_full(full: dict, cfg, device, dtype=torch.bfloat16) -> dict:
+    """Loaded layout from a name -> tensor dict under the checkpoint's names."""
+    w = {"embed": full["embed"].to(dtype).to(device), "lm_head": full["head"].to(dtype).to(device),
+         "final_norm": full["final.norm"].float().to(device), "vocab_start": 0, "layers": [],
+         "full": full}
+    for i, ly in enumerate(cfg.layers):
+        pre = f"l{i}."
+        w["layers"].append(_assemble_layer(lambda k: full[pre + k], ly, lambda k: pre + k in full,
+                                           dtype, device))
+    return w

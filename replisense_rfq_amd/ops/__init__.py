@@ -998,3 +998,98 @@ def reset_plans() -> None:
               _ROPE_PLAN, _SPLIT_PLAN):
         d.clear()
     _TUNED_MS.clear()
+
+
+# ---------------------------------------------------------------------------
+# Ops of the layer-list models (csrc/kernels/mix_*.hip, library _C_mix.so).  The
+# residual stream and every norm are fp32; activations that feed matrix products
+# have the model's dtype (bf16, or fp32 for a model served in full precision).
+def matmul_nt(x, w, out_dtype=None):
+    """x[M, K] . w[N, K]^T on the vendor library (fp32 accumulation; true fp32 for fp32
+    operands); ``out_dtype`` float32 keeps the accumulator's precision for bf16 operands."""
+    if out_dtype is None or out_dtype == x.dtype:
+        return x @ w.t()
+    if x.shape[0] == 0:
+        return torch.empty((0, w.shape[0]), dtype=out_dtype, device=x.device)
+    if x.is_cuda:
+        try:
+            return torch.mm(x, w.t(), out_dtype=out_dtype)
+        except (TypeError, RuntimeError):
+            pass
+    return x.to(out_dtype) @ w.to(out_dtype).t()
+
+
+def embed_sinusoid(ids, positions, table, scale: float, out=None):
+    out = torch.empty((ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device) \
+        if out is None else out
+    if _gpu(table):
+        _native.mix_ops().embed_sinusoid(ids, positions, table, float(scale), out)
+    else:
+        ref.embed_sinusoid(ids, positions, table, scale, out)
+    return out
+
+
+def sandwich_norm(y, residual, w_post, gain, w_pre, eps: float, out=None):
+    """residual (fp32, in place) += rms(y) * w_post * gain, unless y is None; returns
+    rms(residual) * w_pre in fp32."""
+    out = torch.empty_like(residual) if out is None else out
+    if _gpu(residual):
+        _native.mix_ops().sandwich_norm(y, residual, w_post, gain, w_pre, float(eps), out)
+    else:
+        ref.sandwich_norm(y, residual, w_post, gain, w_pre, eps, out)
+    return out
+
+
+def canon_conv(h, w, state, row_state, row_back, row_fwd, positions, out):
+    if _gpu(h):
+        _native.mix_ops().canon_conv(h, w, state, row_state, row_back, row_fwd, positions, out)
+    else:
+        ref.canon_conv(h, w, state, row_state, row_back, row_fwd, positions, out)
+    return out
+
+
+def head_norm_append(qkv, q_w, k_w, eps, slot_mapping, k_cache, v_cache, H, G, dim, vdim, qn,
+                     talk_scaled, qmix, mix_from: int):
+    if _gpu(qkv):
+        _native.mix_ops().head_norm_append(qkv, q_w, k_w, float(eps), slot_mapping, k_cache,
+                                           v_cache, H, G, dim, vdim, qn, talk_scaled, qmix,
+                                           int(mix_from))
+    else:
+        ref.head_norm_append(qkv, q_w, k_w, eps, slot_mapping, k_cache, v_cache, H, G, dim, vdim,
+                             qn, talk_scaled, qmix, mix_from)
+
+
+def attn_talk_decode(qn, k_cache, v_cache, block_tables, q_start, q_len, kv_len, out, slopes,
+                     talk, sink, scale: float, chunk: int):
+    if _gpu(qn):
+        _native.mix_ops().attn_talk_decode(qn, k_cache, v_cache, block_tables, q_start, q_len,
+                                           kv_len, out, slopes, talk, sink, float(scale),
+                                           int(chunk))
+    else:
+        ref.attn_talk_decode(qn, k_cache, v_cache, block_tables, q_start, q_len, kv_len, out,
+                             slopes, talk, sink, scale, chunk)
+
+
+MIXQ_QBLK = 32       # queries per prefill work item of attn_mixq_prefill
+
+
+def attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len, kv_len, work_seq,
+                      work_qblk, out, slopes, sink, chunk: int, qblk: int = MIXQ_QBLK):
+    if _gpu(qmix):
+        _native.mix_ops().attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len,
+                                            kv_len, work_seq, work_qblk, out, slopes, sink,
+                                            int(chunk), int(qblk))
+    else:
+        ref.attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len, kv_len, out,
+                              slopes, sink, chunk)
+
+
+def glu_clamped(gate_up, limit: float, alpha: float = 1.702, out=None):
+    F = gate_up.shape[1] // 2
+    out = torch.empty((gate_up.shape[0], F), dtype=gate_up.dtype, device=gate_up.device) \
+        if out is None else out
+    if _gpu(gate_up):
+        _native.mix_ops().glu_clamped(gate_up, float(limit), float(alpha), out)
+    else:
+        ref.glu_clamped(gate_up, limit, alpha, out)
+    return out

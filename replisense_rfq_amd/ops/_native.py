@@ -63,3 +63,32 @@ def require() -> None:
 def ops():
     require()
     return torch.ops.rfq_amd
+
+
+# The layer-list models' kernels live in a library of their own (``_C_mix.so``:
+# csrc/kernels/mix_*.hip), so that serving such a model compiles and loads only them.
+_MIX_LIB = _LIB.with_name("_C_mix.so")
+_mix_loaded = False
+_mix_error: Exception | None = None
+
+
+def mix_ops():
+    """torch.ops.rfq_mix, building the library on first use if it is not there."""
+    global _mix_loaded, _mix_error
+    if not _mix_loaded:
+        with _lock:
+            if not _mix_loaded:
+                try:
+                    if not _MIX_LIB.exists() and os.environ.get("RFQ_AUTOBUILD", "1") == "1":
+                        from .. import _build
+
+                        _build.build_mix_kernels()
+                    torch.ops.load_library(str(_MIX_LIB))
+                    _mix_loaded = True
+                except Exception as e:
+                    _mix_error = e
+    if not _mix_loaded:
+        raise RuntimeError(
+            f"replisense_rfq_amd native op library unavailable ({_MIX_LIB}): {_mix_error!r}. "
+            "Run `python -c 'import __graft_entry__ as g; g.build()'` (hipcc, gfx950).")
+    return torch.ops.rfq_mix

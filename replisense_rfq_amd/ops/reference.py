@@ -181,3 +181,177 @@ def moe_forward(x, w13, w2, router_logits, topk: int, expert_offset: int = 0):
 
 def softmax_scale(head_dim: int = 128) -> float:
     return 1.0 / math.sqrt(head_dim)
+
+
+# --------------------------------------------------------------------------
+# Ops of the layer-list models (fp32 residual stream, sandwich norms, short causal
+# input convolutions with per-sequence state, biased / mixed-head / sink attention).
+def embed_sinusoid(ids, positions, table, scale: float, out) -> None:
+    """out[t] = table[ids[t]] * scale + pe(positions[t]) in fp32, with
+    pe[2i] = sin(p * 10000^(-2i/d)), pe[2i+1] = cos of the same angle."""
+    d = table.shape[1]
+    x = table[ids.long()].float() * scale
+    i2 = torch.arange(0, d, 2, dtype=torch.float32, device=table.device)
+    inv = torch.pow(torch.tensor(10000.0, device=table.device), -i2 / d)
+    ang = positions.float()[:, None] * inv[None]
+    x[:, 0::2] += torch.sin(ang)[:, : (d + 1) // 2]
+    x[:, 1::2] += torch.cos(ang)[:, : d // 2]
+    out.copy_(x)
+
+
+def _rms(x, eps):
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+
+def sandwich_norm(y, residual, w_post, gain, w_pre, eps: float, out) -> None:
+    """residual += rms(y) * w_post * gain (skipped when y is None); out = rms(residual) * w_pre."""
+    if y is not None:
+        residual.add_(_rms(y.float(), eps) * w_post.float() * gain.float())
+    out.copy_(_rms(residual, eps) * w_pre.float())
+
+
+def canon_conv(h, w, state, row_state, row_back, row_fwd, positions, out) -> None:
+    """out[t] = h[t] + sum_j w[:, j] h[t - (taps-1-j)] over the sequence of row t; inputs
+    before the scheduled run come from the sequence's state half (its last taps-1
+    inputs), inputs before position 0 are zero.  The other half receives the run's last
+    taps-1 inputs.  state: [2 * slots, taps-1, d] fp32; row_state = slot * 2 + read half."""
+    T, d = h.shape
+    taps = w.shape[1]
+    K = taps - 1
+    S = state.shape[0] // 2
+    hf = h.float()
+    wf = w.float()
+    acc = hf.clone()
+    new = {}
+    for t in range(T):
+        code, i, f, p = int(row_state[t]), int(row_back[t]), int(row_fwd[t]), int(positions[t])
+        rd = (code & 1) * S + (code >> 1) if code >= 0 else -1
+        for dl in range(taps):                      # delay dl uses tap j = taps-1-dl
+            if dl == 0:
+                src = hf[t]
+            elif dl <= i:
+                src = hf[t - dl]
+            elif p - dl >= 0 and rd >= 0:
+                src = state[rd, K + i - dl]
+            else:
+                continue
+            acc[t] += wf[:, taps - 1 - dl] * src
+        if code >= 0:
+            wr = (1 - (code & 1)) * S + (code >> 1)
+            q = i + f + 1
+            if f < K:
+                new[(wr, K - 1 - f)] = hf[t]
+            if i == 0:
+                for e in range(0, K - q):            # run shorter than the state: shift
+                    new[(wr, e)] = state[rd, e + q].clone()
+    for (wr, e), v in new.items():
+        state[wr, e] = v
+    out.copy_(acc.to(out.dtype))
+
+
+def head_norm_append(qkv, q_w, k_w, eps: float, slot_mapping, k_cache, v_cache, H: int, G: int,
+                     dim: int, vdim: int, qn, talk_scaled, qmix, mix_from: int) -> None:
+    """Per head: q <- rms(q) * q_w (into qn, fp32), k <- rms(k) * k_w and v <- v / rms(v)
+    into the paged caches [blocks, G, BS, dim | vdim].  Rows >= mix_from also get mixed
+    queries qmix[t - mix_from, h, c*dim:(c+1)*dim] = sum_{g in group c} talk_scaled[h, g] qn[t, g]
+    (talk_scaled = score scale * head-mixing matrix), so that mixed scores are one product
+    with the concatenated key heads."""
+    T = qkv.shape[0]
+    if T == 0:
+        return
+    BS = k_cache.shape[2]
+    q = qkv[:, : H * dim].float().view(T, H, dim)
+    k = qkv[:, H * dim:(H + G) * dim].float().view(T, G, dim)
+    v = qkv[:, (H + G) * dim:(H + G) * dim + G * vdim].float().view(T, G, vdim)
+    qf = _rms(q, eps) * q_w.float()
+    qn.copy_(qf)
+    kf = _rms(k, eps) * k_w.float()
+    vf = _rms(v, eps)
+    slots = slot_mapping[:T].long()
+    ok = slots >= 0
+    if ok.any():
+        sl = slots[ok]
+        blk, off = sl // BS, sl % BS
+        k_cache[blk, :, off] = kf[ok].to(k_cache.dtype)
+        v_cache[blk, :, off] = vf[ok].to(v_cache.dtype)
+    if qmix is not None and mix_from < T:
+        rep = H // G
+        ts = talk_scaled.float().view(H, G, rep)
+        qg = qf[mix_from:].view(T - mix_from, G, rep, dim)
+        qmix.copy_(torch.einsum("hcr,tcrd->thcd", ts, qg).reshape(T - mix_from, H, G * dim))
+
+
+def _sink_softmax(s, ok, sink):
+    s = s.masked_fill(~ok, float("-inf"))
+    m = s.max(-1).values
+    if sink is not None:
+        m = torch.maximum(m, sink.float()[:, None])
+    m = torch.where(torch.isinf(m), torch.zeros_like(m), m)
+    e = torch.exp(s - m[..., None])
+    den = e.sum(-1)
+    if sink is not None:
+        den = den + torch.exp(sink.float()[:, None] - m)
+    return e / den.clamp_min(1e-38)[..., None]
+
+
+def attn_talk_decode(qn, k_cache, v_cache, block_tables, q_start, q_len, kv_len, out, slopes,
+                     talk, sink, scale: float, chunk: int) -> None:
+    """Decode / short-extend rows: score_g = scale q_g.k - slopes[g] (i - j), mixed over
+    heads by ``talk`` [H, H] (None = no mixing), masked to j <= i inside i's block of
+    ``chunk`` positions (0 = causal), softmax with a per-head sink logit in the denominator."""
+    H, dim = qn.shape[1], qn.shape[2]
+    G = k_cache.shape[1]
+    rep = H // G
+    for b in range(q_len.shape[0]):
+        ql, kl, t0 = int(q_len[b]), int(kv_len[b]), int(q_start[b])
+        if ql == 0:
+            continue
+        k = _gather_kv(k_cache, block_tables[b], kl).float().repeat_interleave(rep, 0)
+        v = _gather_kv(v_cache, block_tables[b], kl).float().repeat_interleave(rep, 0)
+        q = qn[t0:t0 + ql].permute(1, 0, 2)
+        i = torch.arange(kl - ql, kl, device=qn.device)[:, None]
+        j = torch.arange(kl, device=qn.device)[None, :]
+        s = torch.einsum("hqd,hkd->hqk", q, k) * scale - slopes.float()[:, None, None] * (i - j).float()
+        if talk is not None:
+            s = torch.einsum("hg,gqk->hqk", talk.float(), s)
+        ok = j <= i
+        if chunk > 0:
+            ok = ok & ((i // chunk) == (j // chunk))
+        p = _sink_softmax(s, ok[None], sink)
+        o = torch.einsum("hqk,hkd->qhd", p, v)
+        out[t0:t0 + ql].copy_(o.reshape(ql, -1).to(out.dtype))
+
+
+def attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len, kv_len, out, slopes,
+                      sink, chunk: int) -> None:
+    """Prefill rows on pre-mixed, pre-scaled queries [T, H, G*dim]: every head's score is
+    one product with the concatenation of all G key heads, minus slopes[h] (i - j) (the
+    slopes already mixed); values come from the head's own key/value head."""
+    H = qmix.shape[1]
+    G = k_cache.shape[1]
+    rep = H // G
+    for b in range(q_len.shape[0]):
+        ql, kl, t0 = int(q_len[b]), int(kv_len[b]), int(q_start[b])
+        if ql == 0:
+            continue
+        k = _gather_kv(k_cache, block_tables[b], kl).float()            # [G, kl, dim]
+        kc = k.permute(1, 0, 2).reshape(kl, -1)                          # [kl, G*dim]
+        v = _gather_kv(v_cache, block_tables[b], kl).float().repeat_interleave(rep, 0)
+        i = torch.arange(kl - ql, kl, device=qmix.device)[:, None]
+        j = torch.arange(kl, device=qmix.device)[None, :]
+        s = torch.einsum("qhe,ke->hqk", qmix[t0:t0 + ql].float(), kc)
+        s = s - slopes.float()[:, None, None] * (i - j).float()
+        ok = j <= i
+        if chunk > 0:
+            ok = ok & ((i // chunk) == (j // chunk))
+        p = _sink_softmax(s, ok[None], sink)
+        o = torch.einsum("hqk,hkd->qhd", p, v)
+        out[t0:t0 + ql].copy_(o.reshape(ql, -1).to(out.dtype))
+
+
+def glu_clamped(gate_up, limit: float, alpha: float, out) -> None:
+    """g = min(gate, limit), u = clamp(up, -limit, limit); out = g sigmoid(alpha g) (u + 1)."""
+    F = out.shape[1]
+    g = gate_up[:, :F].float().clamp(max=limit)
+    u = gate_up[:, F:].float().clamp(-limit, limit)
+    out.copy_((g * torch.sigmoid(alpha * g) * (u + 1)).to(out.dtype))

@@ -29,6 +29,7 @@ class EngineConfig:
     dp: int = 1
     device: str = "auto"                 # auto -> cuda if available else cpu
     seed: int = 0
+    dtype: str = "bfloat16"              # float32: layer-list models only (full-precision serving)
     kv_fraction: float = 0.85            # of free HBM for the paged KV pool (bench.py default)
     max_kv_blocks: int = 0               # 0 = from kv_fraction
     block_size: int = 32                 # tokens per KV page (kernel tile)
@@ -71,6 +72,7 @@ class EngineConfig:
             dp=_env("RFQ_DP", cls.dp, int),
             device=_env("RFQ_DEVICE", cls.device),
             seed=_env("RFQ_SEED", cls.seed, int),
+            dtype=_env("RFQ_DTYPE", cls.dtype),
             kv_fraction=_env("RFQ_KV_FRACTION", cls.kv_fraction, float),
             max_num_seqs=_env("RFQ_MAX_BATCH", cls.max_num_seqs, int),
             max_batched_tokens=_env("RFQ_PREFILL_CHUNK", cls.max_batched_tokens, int),
