@@ -1,0 +1,245 @@
+// torch op registrations of the layer-list models' kernels (namespace torch.ops.rfq_mix).
+//
+// Every op launches on the caller's current HIP stream, allocates nothing and never
+// synchronises, so a decode step can be captured into a hipGraph.  Shapes are checked on the
+// host against what the kernels index before anything is launched.
+#include <torch/library.h>
+#include <ATen/ATen.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rfqmix {
+void launch_embed_sinusoid(bool, const int32_t*, const int32_t*, const void*, const float*, float,
+                           float*, int, int, int, hipStream_t);
+void launch_sandwich_norm(bool, const void*, int64_t, float*, const float*, const float*,
+                          const float*, float*, int, int, float, hipStream_t);
+void launch_canon_conv(bool, const float*, const float*, float*, const int32_t*, const int32_t*,
+                       const int32_t*, const int32_t*, void*, int, int, int, int, hipStream_t);
+void launch_head_norm_append(bool, const void*, int64_t, const float*, const float*, float,
+                             const int32_t*, void*, void*, int, int, int, int, int, int, float*,
+                             const float*, float*, int, hipStream_t);
+void launch_glu_clamped(bool, const void*, int64_t, void*, int64_t, int, int, float, float,
+                        hipStream_t);
+int launch_attn_talk_decode(bool, const float*, const void*, const void*, const int32_t*, int,
+                            const int32_t*, const int32_t*, const int32_t*, void*, int64_t,
+                            const float*, const float*, const float*, float, int, int, int, int,
+                            int, int, int, int, hipStream_t);
+bool launch_attn_mixq_prefill(bool, const float*, const void*, const void*, const int32_t*, int,
+                              const int32_t*, const int32_t*, const int32_t*, const int32_t*,
+                              const int32_t*, int, void*, int64_t, const float*, const float*, int,
+                              int, int, int, int, int, hipStream_t);
+bool launch_attn_mixq_prefill_mfma(const float*, const void*, const void*, const int32_t*, int,
+                                   const int32_t*, const int32_t*, const int32_t*, const int32_t*,
+                                   const int32_t*, int, void*, int64_t, const float*, const float*,
+                                   int, int, int, int, int, int, hipStream_t);
+}  // namespace rfqmix
+
+namespace {
+
+using at::Tensor;
+using OptT = c10::optional<Tensor>;
+
+hipStream_t stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+bool act_f32(const Tensor& t, const char* what) {
+  TORCH_CHECK(t.is_cuda(), what, ": not a GPU tensor");
+  TORCH_CHECK(t.scalar_type() == at::kFloat || t.scalar_type() == at::kBFloat16, what,
+              ": float32 or bfloat16 expected");
+  return t.scalar_type() == at::kFloat;
+}
+
+const float* f32p(const Tensor& t, const char* what, int64_t numel = -1) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous(), what,
+              ": contiguous float32 GPU tensor expected");
+  TORCH_CHECK(numel < 0 || t.numel() == numel, what, ": wrong size");
+  return t.data_ptr<float>();
+}
+
+const int32_t* i32p(const Tensor& t, const char* what, int64_t min_numel) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), what,
+              ": contiguous int32 GPU tensor expected");
+  TORCH_CHECK(t.numel() >= min_numel, what, ": too short");
+  return t.data_ptr<int32_t>();
+}
+
+const float* optf(const OptT& t, const char* what, int64_t numel) {
+  return t.has_value() ? f32p(*t, what, numel) : nullptr;
+}
+
+void embed_sinusoid(const Tensor& ids, const Tensor& pos, const Tensor& table,
+                    const Tensor& inv_freq, double scale, const Tensor& out) {
+  const bool f32 = act_f32(table, "embed_sinusoid table");
+  const int T = (int)ids.numel(), d = (int)table.size(1);
+  TORCH_CHECK(table.dim() == 2 && table.is_contiguous(), "embed_sinusoid: table [V, d]");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == d, "embed_sinusoid: out [T, d]");
+  rfqmix::launch_embed_sinusoid(f32, i32p(ids, "ids", T), i32p(pos, "positions", T),
+                                table.data_ptr(), f32p(inv_freq, "inv_freq", (d + 1) / 2),
+                                (float)scale, const_cast<float*>(f32p(out, "out")), T, d,
+                                (int)table.size(0), stream());
+}
+
+void sandwich_norm(const OptT& y, const Tensor& residual, const OptT& w_post, const OptT& gain,
+                   const Tensor& w_pre, double eps, const Tensor& out) {
+  TORCH_CHECK(residual.dim() == 2, "sandwich_norm: residual [T, d]");
+  const int T = (int)residual.size(0), d = (int)residual.size(1);
+  bool f32 = true;
+  const void* yp = nullptr;
+  int64_t ys = 0;
+  if (y.has_value()) {
+    f32 = act_f32(*y, "sandwich_norm y");
+    TORCH_CHECK(y->dim() == 2 && y->size(0) == T && y->size(1) == d && y->stride(1) == 1,
+                "sandwich_norm: y [T, d]");
+    TORCH_CHECK(w_post.has_value() && gain.has_value(), "sandwich_norm: y needs w_post and gain");
+    yp = y->data_ptr();
+    ys = y->stride(0);
+  }
+  TORCH_CHECK(out.sizes() == residual.sizes(), "sandwich_norm: out [T, d]");
+  rfqmix::launch_sandwich_norm(f32, yp, ys, const_cast<float*>(f32p(residual, "residual")),
+                               y.has_value() ? f32p(*w_post, "w_post", d) : nullptr,
+                               y.has_value() ? f32p(*gain, "gain", d) : nullptr,
+                               f32p(w_pre, "w_pre", d), const_cast<float*>(f32p(out, "out")), T, d,
+                               (float)eps, stream());
+}
+
+void canon_conv(const Tensor& h, const Tensor& w, const Tensor& state, const Tensor& row_state,
+                const Tensor& row_back, const Tensor& row_fwd, const Tensor& pos,
+                const Tensor& out) {
+  TORCH_CHECK(h.dim() == 2 && w.dim() == 2 && state.dim() == 3, "canon_conv: h [T, d], w [d, taps], state [2S, taps-1, d]");
+  const int T = (int)h.size(0), d = (int)h.size(1), taps = (int)w.size(1);
+  TORCH_CHECK(w.size(0) == d && taps >= 1, "canon_conv: w [d, taps]");
+  TORCH_CHECK(state.size(1) == taps - 1 && state.size(2) == d && state.size(0) % 2 == 0,
+              "canon_conv: state [2 * slots, taps - 1, d]");
+  const bool f32 = act_f32(out, "canon_conv out");
+  TORCH_CHECK(out.is_contiguous() && out.size(0) == T && out.size(1) == d, "canon_conv: out [T, d]");
+  rfqmix::launch_canon_conv(f32, f32p(h, "h"), f32p(w, "w"), const_cast<float*>(f32p(state, "state")),
+                            i32p(row_state, "row_state", T), i32p(row_back, "row_back", T),
+                            i32p(row_fwd, "row_fwd", T), i32p(pos, "positions", T), out.data_ptr(),
+                            T, d, taps, (int)state.size(0) / 2, stream());
+}
+
+void head_norm_append(const Tensor& qkv, const Tensor& q_w, const Tensor& k_w, double eps,
+                      const Tensor& slots, const Tensor& k_cache, const Tensor& v_cache, int64_t H,
+                      int64_t G, int64_t dim, int64_t vdim, const Tensor& qn, const OptT& ts,
+                      const OptT& qmix, int64_t mix_from) {
+  const bool f32 = act_f32(qkv, "head_norm_append qkv");
+  const int T = (int)qkv.size(0);
+  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && qkv.size(1) == H * dim + G * (dim + vdim),
+              "head_norm_append: qkv [T, H dim + G (dim + vdim)]");
+  TORCH_CHECK(H % G == 0 && H * dim * 4 <= 64 * 1024, "head_norm_append: heads do not fit");
+  TORCH_CHECK(k_cache.scalar_type() == qkv.scalar_type() && v_cache.scalar_type() == qkv.scalar_type(),
+              "head_norm_append: cache dtype");
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() && k_cache.size(1) == G &&
+              k_cache.size(3) == dim, "head_norm_append: k_cache [blocks, G, BS, dim]");
+  TORCH_CHECK(v_cache.dim() == 4 && v_cache.is_contiguous() && v_cache.size(1) == G &&
+              v_cache.size(3) == vdim && v_cache.size(2) == k_cache.size(2) &&
+              v_cache.size(0) == k_cache.size(0), "head_norm_append: v_cache [blocks, G, BS, vdim]");
+  float* qm = nullptr;
+  if (qmix.has_value() && mix_from < T) {
+    TORCH_CHECK(ts.has_value(), "head_norm_append: mixing needs the matrix");
+    qm = const_cast<float*>(f32p(*qmix, "qmix", (int64_t)(T - mix_from) * H * G * dim));
+  }
+  rfqmix::launch_head_norm_append(
+      f32, qkv.data_ptr(), qkv.stride(0), f32p(q_w, "q_w", dim), f32p(k_w, "k_w", dim), (float)eps,
+      i32p(slots, "slot_mapping", T), k_cache.data_ptr(), v_cache.data_ptr(), T, (int)H, (int)G,
+      (int)dim, (int)vdim, (int)k_cache.size(2), const_cast<float*>(f32p(qn, "qn", (int64_t)T * H * dim)),
+      optf(ts, "talk_scaled", H * H), qm, (int)mix_from, stream());
+}
+
+void attn_talk_decode(const Tensor& qn, const Tensor& k_cache, const Tensor& v_cache,
+                      const Tensor& bt, const Tensor& q_start, const Tensor& q_len,
+                      const Tensor& kv_len, const Tensor& out, const Tensor& slopes,
+                      const OptT& talk, const OptT& sink, double scale, int64_t chunk,
+                      int64_t max_rows) {
+  const bool f32 = act_f32(k_cache, "attn_talk_decode k_cache");
+  TORCH_CHECK(qn.dim() == 3, "attn_talk_decode: qn [T, H, dim]");
+  const int H = (int)qn.size(1), dim = (int)qn.size(2), G = (int)k_cache.size(1);
+  const int vdim = (int)v_cache.size(3), BS = (int)k_cache.size(2), NA = (int)q_len.numel();
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() &&
+              v_cache.is_contiguous() && k_cache.size(3) == dim && v_cache.size(1) == G &&
+              v_cache.size(2) == BS && v_cache.scalar_type() == k_cache.scalar_type() && H % G == 0,
+              "attn_talk_decode: caches [blocks, G, BS, dim | vdim]");
+  TORCH_CHECK(out.scalar_type() == k_cache.scalar_type() && out.dim() == 2 &&
+              out.size(0) == qn.size(0) && out.size(1) == (int64_t)H * vdim && out.stride(1) == 1,
+              "attn_talk_decode: out [T, H vdim]");
+  TORCH_CHECK(bt.dim() == 2 && bt.size(0) == NA, "attn_talk_decode: block_tables [NA, maxb]");
+  TORCH_CHECK(max_rows >= 1 && max_rows <= 65535, "attn_talk_decode: max_rows");
+  const int kt = rfqmix::launch_attn_talk_decode(
+      f32, f32p(qn, "qn"), k_cache.data_ptr(), v_cache.data_ptr(), i32p(bt, "block_tables", 0),
+      (int)bt.size(1), i32p(q_start, "q_start", NA), i32p(q_len, "q_len", NA),
+      i32p(kv_len, "kv_len", NA), out.data_ptr(), out.stride(0), f32p(slopes, "slopes", H),
+      optf(talk, "talk", (int64_t)H * H), optf(sink, "sink", H), (float)scale, (int)chunk, NA,
+      (int)max_rows, H, G, dim, vdim, BS, stream());
+  TORCH_CHECK(kt > 0, "attn_talk_decode: head sizes do not fit the LDS");
+}
+
+void attn_mixq_prefill(const Tensor& qmix, const Tensor& k_cache, const Tensor& v_cache,
+                       const Tensor& bt, const Tensor& q_start, const Tensor& q_len,
+                       const Tensor& kv_len, const Tensor& work_seq, const Tensor& work_qblk,
+                       const Tensor& out, const Tensor& slopes, const OptT& sink, int64_t chunk,
+                       int64_t qblk, int64_t mfma) {
+  const bool f32 = act_f32(k_cache, "attn_mixq_prefill k_cache");
+  TORCH_CHECK(qmix.dim() == 3, "attn_mixq_prefill: qmix [T, H, G dim]");
+  const int H = (int)qmix.size(1), G = (int)k_cache.size(1), dim = (int)k_cache.size(3);
+  const int vdim = (int)v_cache.size(3), BS = (int)k_cache.size(2), NB = (int)q_len.numel();
+  const int W = (int)work_seq.numel();
+  TORCH_CHECK(qblk == 32, "attn_mixq_prefill: 32 queries per work item");
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() &&
+              v_cache.is_contiguous() && qmix.size(2) == (int64_t)G * dim && v_cache.size(1) == G &&
+              v_cache.size(2) == BS && v_cache.scalar_type() == k_cache.scalar_type() && H % G == 0,
+              "attn_mixq_prefill: caches [blocks, G, BS, dim | vdim], qmix [T, H, G dim]");
+  TORCH_CHECK(out.scalar_type() == k_cache.scalar_type() && out.dim() == 2 &&
+              out.size(0) == qmix.size(0) && out.size(1) == (int64_t)H * vdim && out.stride(1) == 1,
+              "attn_mixq_prefill: out [T, H vdim]");
+  TORCH_CHECK(bt.dim() == 2 && bt.size(0) == NB, "attn_mixq_prefill: block_tables [NB, maxb]");
+  const float* sk = optf(sink, "sink", H);
+  if (mfma && !f32) {
+    const bool ok = rfqmix::launch_attn_mixq_prefill_mfma(
+        f32p(qmix, "qmix"), k_cache.data_ptr(), v_cache.data_ptr(), i32p(bt, "block_tables", 0),
+        (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
+        i32p(kv_len, "kv_len", NB), i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W),
+        W, out.data_ptr(), out.stride(0), f32p(slopes, "slopes", H), sk, (int)chunk, H, G, dim,
+        vdim, BS, stream());
+    if (ok) return;
+  }
+  const bool ok = rfqmix::launch_attn_mixq_prefill(
+      f32, f32p(qmix, "qmix"), k_cache.data_ptr(), v_cache.data_ptr(), i32p(bt, "block_tables", 0),
+      (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
+      i32p(kv_len, "kv_len", NB), i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W), W,
+      out.data_ptr(), out.stride(0), f32p(slopes, "slopes", H), sk, (int)chunk, H, G, dim, vdim, BS,
+      stream());
+  TORCH_CHECK(ok, "attn_mixq_prefill: value size does not fit the LDS");
+}
+
+void glu_clamped(const Tensor& gu, double limit, double alpha, const Tensor& out) {
+  const bool f32 = act_f32(gu, "glu_clamped gate_up");
+  const int T = (int)gu.size(0), F = (int)out.size(1);
+  TORCH_CHECK(gu.dim() == 2 && out.dim() == 2 && gu.size(1) == 2 * F && out.size(0) == T &&
+              gu.stride(1) == 1 && out.stride(1) == 1 && out.scalar_type() == gu.scalar_type(),
+              "glu_clamped: gate_up [T, 2F], out [T, F]");
+  TORCH_CHECK((F + 255) / 256 <= 65535, "glu_clamped: F too large");
+  rfqmix::launch_glu_clamped(f32, gu.data_ptr(), gu.stride(0), out.data_ptr(), out.stride(0), T, F,
+                             (float)limit, (float)alpha, stream());
+}
+
+}  // namespace
+
+TORCH_LIBRARY(rfq_mix, m) {
+  m.def("embed_sinusoid(Tensor ids, Tensor pos, Tensor table, Tensor inv_freq, float scale, Tensor(a!) out) -> ()");
+  m.def("sandwich_norm(Tensor? y, Tensor(a!) residual, Tensor? w_post, Tensor? gain, Tensor w_pre, float eps, Tensor(b!) out) -> ()");
+  m.def("canon_conv(Tensor h, Tensor w, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor(b!) out) -> ()");
+  m.def("head_norm_append(Tensor qkv, Tensor q_w, Tensor k_w, float eps, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, int H, int G, int dim, int vdim, Tensor(c!) qn, Tensor? ts, Tensor(d!)? qmix, int mix_from) -> ()");
+  m.def("attn_talk_decode(Tensor qn, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor(a!) out, Tensor slopes, Tensor? talk, Tensor? sink, float scale, int chunk, int max_rows) -> ()");
+  m.def("attn_mixq_prefill(Tensor qmix, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor slopes, Tensor? sink, int chunk, int qblk, int mfma) -> ()");
+  m.def("glu_clamped(Tensor gate_up, float limit, float alpha, Tensor(a!) out) -> ()");
+}
+
+TORCH_LIBRARY_IMPL(rfq_mix, CUDA, m) {
+  m.impl("embed_sinusoid", &embed_sinusoid);
+  m.impl("sandwich_norm", &sandwich_norm);
+  m.impl("canon_conv", &canon_conv);
+  m.impl("head_norm_append", &head_norm_append);
+  m.impl("attn_talk_decode", &attn_talk_decode);
+  m.impl("attn_mixq_prefill", &attn_mixq_prefill);
+  m.impl("glu_clamped", &glu_clamped);
+}

@@ -64,6 +64,7 @@ class LivisunLM:
         self.kv_k = self.kv_v = None
         self.state = None
         self.norms_folded = False
+        self.inv_freq = ops.sinusoid_inv_freq(cfg.hidden, self.device)
         if dtype == torch.float32:
             torch.backends.cuda.matmul.allow_tf32 = False
         for ly, lw in zip(cfg.layers, self.w["layers"]):
@@ -101,7 +102,7 @@ class LivisunLM:
         dt, dev = self.dtype, self.device
         rs, rb, rf = m.extra["row_state"], m.extra["row_back"], m.extra["row_fwd"]
         pos = m.positions[:T]
-        x = ops.embed_sinusoid(m.input_ids[:T], pos, w["embed"], cfg.embed_scale)
+        x = ops.embed_sinusoid(m.input_ids[:T], pos, w["embed"], self.inv_freq, cfg.embed_scale)
         h = ops.sandwich_norm(None, x, None, None, w["layers"][0]["norm1"], eps)
         hc = torch.empty((T, cfg.hidden), dtype=dt, device=dev)
         L = cfg.n_layers

@@ -1019,13 +1019,19 @@ def matmul_nt(x, w, out_dtype=None):
     return x.to(out_dtype) @ w.to(out_dtype).t()
 
 
-def embed_sinusoid(ids, positions, table, scale: float, out=None):
+def sinusoid_inv_freq(d: int, device, base: float = 10000.0):
+    """inv_freq[i] = base^(-2i/d), fp32: the angle of entries 2i (sin) and 2i+1 (cos)."""
+    i2 = torch.arange(0, d, 2, dtype=torch.float32, device=device)
+    return torch.pow(torch.tensor(base, dtype=torch.float32, device=device), -i2 / d).contiguous()
+
+
+def embed_sinusoid(ids, positions, table, inv_freq, scale: float, out=None):
     out = torch.empty((ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device) \
         if out is None else out
     if _gpu(table):
-        _native.mix_ops().embed_sinusoid(ids, positions, table, float(scale), out)
+        _native.mix_ops().embed_sinusoid(ids, positions, table, inv_freq, float(scale), out)
     else:
-        ref.embed_sinusoid(ids, positions, table, scale, out)
+        ref.embed_sinusoid(ids, positions, table, inv_freq, scale, out)
     return out
 
 
@@ -1059,18 +1065,22 @@ def head_norm_append(qkv, q_w, k_w, eps, slot_mapping, k_cache, v_cache, H, G, d
                              qn, talk_scaled, qmix, mix_from)
 
 
+TALK_DECODE_MAX_ROWS = 32      # rows per sequence of the decode section (the runner's EXT_MAX)
+
+
 def attn_talk_decode(qn, k_cache, v_cache, block_tables, q_start, q_len, kv_len, out, slopes,
-                     talk, sink, scale: float, chunk: int):
+                     talk, sink, scale: float, chunk: int, max_rows: int = TALK_DECODE_MAX_ROWS):
     if _gpu(qn):
         _native.mix_ops().attn_talk_decode(qn, k_cache, v_cache, block_tables, q_start, q_len,
                                            kv_len, out, slopes, talk, sink, float(scale),
-                                           int(chunk))
+                                           int(chunk), int(max_rows))
     else:
         ref.attn_talk_decode(qn, k_cache, v_cache, block_tables, q_start, q_len, kv_len, out,
                              slopes, talk, sink, scale, chunk)
 
 
 MIXQ_QBLK = 32       # queries per prefill work item of attn_mixq_prefill
+MIXQ_MFMA = os.environ.get("RFQ_MIXQ_MFMA", "1") != "0"     # bf16: MFMA tiles where sizes fit
 
 
 def attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len, kv_len, work_seq,
@@ -1078,7 +1088,7 @@ def attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len, kv_l
     if _gpu(qmix):
         _native.mix_ops().attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len,
                                             kv_len, work_seq, work_qblk, out, slopes, sink,
-                                            int(chunk), int(qblk))
+                                            int(chunk), int(qblk), int(MIXQ_MFMA))
     else:
         ref.attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len, kv_len, out,
                               slopes, sink, chunk)

@@ -186,14 +186,12 @@ def softmax_scale(head_dim: int = 128) -> float:
 # --------------------------------------------------------------------------
 # Ops of the layer-list models (fp32 residual stream, sandwich norms, short causal
 # input convolutions with per-sequence state, biased / mixed-head / sink attention).
-def embed_sinusoid(ids, positions, table, scale: float, out) -> None:
+def embed_sinusoid(ids, positions, table, inv_freq, scale: float, out) -> None:
     """out[t] = table[ids[t]] * scale + pe(positions[t]) in fp32, with
-    pe[2i] = sin(p * 10000^(-2i/d)), pe[2i+1] = cos of the same angle."""
+    pe[2i] = sin(p * inv_freq[i]), pe[2i+1] = cos of the same angle."""
     d = table.shape[1]
     x = table[ids.long()].float() * scale
-    i2 = torch.arange(0, d, 2, dtype=torch.float32, device=table.device)
-    inv = torch.pow(torch.tensor(10000.0, device=table.device), -i2 / d)
-    ang = positions.float()[:, None] * inv[None]
+    ang = positions.float()[:, None] * inv_freq.float()[None]
     x[:, 0::2] += torch.sin(ang)[:, : (d + 1) // 2]
     x[:, 1::2] += torch.cos(ang)[:, : d // 2]
     out.copy_(x)
