@@ -1,0 +1,101 @@
+"""Small Livisun models, engines around them and a schedule driver for the tests."""
+import torch
+
+from replisense_rfq_amd.engine.engine import LLMEngine
+from replisense_rfq_amd.models.config import LayeredConfig
+from replisense_rfq_amd.models.livisun import LivisunLM
+from replisense_rfq_amd.models.weights import init_layered_weights, layered_from_full
+from replisense_rfq_amd.utils.config import EngineConfig
+
+from . import oracle
+
+
+def layer(heads, kv_heads, dim, vdim, chunk, ff, scale=0.3, limit=1.5):
+    return {"type": "attention",
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                      "scale": scale, "mask": {"size": chunk}},
+            "mlp": None if ff is None else {"kind": "dense", "ff": ff, "limit": limit}}
+
+
+def config(layers, vocab=61, width=48, taps=3, emb=2.5, eps=1e-5):
+    return {"architecture": "Livisun", "vocab": vocab, "width": width, "layers": layers,
+            "norm": {"eps": eps}, "embedding": {"scale": emb}, "canon": {"taps": taps}}
+
+
+# sizes unlike each other: dim != vdim, H = 3G / G = 1 / G = H, a layer without feed-forward,
+# blocks that are no multiple of the 32-token page, 2 and 4 taps
+SMALL = config([layer(6, 2, 16, 8, 7, 40), layer(2, 1, 24, 24, 20, None), layer(3, 3, 8, 16, 45, 24)])
+TAPS4 = config([layer(4, 2, 8, 8, 11, 32, scale=0.5, limit=0.7), layer(4, 4, 16, 8, 64, 16)],
+               width=40, taps=4, emb=1.0)
+TAPS2 = config([layer(2, 2, 32, 16, 33, 56)], width=64, taps=2, emb=7.0, eps=1e-3)
+TAPS1 = config([layer(4, 1, 16, 16, 5, 24)], width=32, taps=1)
+
+
+def build(cfg_dict, device="cpu", dtype=torch.float32, seed=0, full=None, **eng_kw):
+    cfg = LayeredConfig.from_json(cfg_dict, name="test-livisun")
+    w = init_layered_weights(cfg, device, dtype, seed) if full is None \
+        else layered_from_full(full, cfg, device, dtype)
+    model = LivisunLM(cfg, device, weights=w, dtype=dtype)
+    kw = dict(model="tiny-livisun", device=str(device), max_num_seqs=4, max_kv_blocks=24,
+              max_batched_tokens=512, max_model_len=512, use_graphs=False, grammar=False,
+              prefix_cache=False, warm_prefix=False, tune_gemm=False, jump_forward=False,
+              dtype="float32" if dtype == torch.float32 else "bfloat16")
+    kw.update(eng_kw)
+    eng = LLMEngine(EngineConfig(**kw), model=model)
+    return eng, w["full"]
+
+
+def run_schedule(eng, steps):
+    """steps: list of {"entries": [(name, tokens, want offsets)], "end": [names]}.
+    Returns {(name, absolute position): logits row (fp32, cpu)}."""
+    live, out = {}, {}
+    for st in steps:
+        for name, toks, want in st["entries"]:
+            seq = live.get(name)
+            base = len(seq.tokens) if seq is not None else 0
+            want = [base + w for w in want]
+            if seq is None:
+                live[name] = eng.score_request(list(toks), want)
+            else:
+                eng.score_extend(seq, list(toks), want)
+        got = eng.score_step()
+        assert eng.core.num_waiting == 0, "a request of the step was not admitted"
+        if got is not None:
+            rows, logits = got
+            names = {s.core_id: n for n, s in live.items()}
+            for (s, p), row in zip(rows, logits.float().cpu()):
+                out[(names[s.core_id], p)] = row
+        for name in st.get("end", []):
+            eng.abort_request(live.pop(name), "stop")
+    return out
+
+
+def alone(tokens, cuts, name="a"):
+    """One request cut into portions of the given sizes (the rest in one), every position wanted."""
+    steps, at = [], 0
+    for c in list(cuts) + [len(tokens)]:
+        c = min(c, len(tokens) - at)
+        if c <= 0:
+            break
+        steps.append({"entries": [(name, tokens[at:at + c], list(range(c)))], "end": []})
+        at += c
+    steps[-1]["end"] = [name]
+    return steps
+
+
+def check(got, cfg_dict, full, requests, tol=2e-4):
+    """Every produced row against the oracle's logits of that request and position."""
+    worst = 0.0
+    ref = {n: oracle.forward(cfg_dict, full, t) for n, t in requests.items()}
+    assert got, "no logits produced"
+    for (n, p), row in got.items():
+        r = ref[n][p]
+        err = float((row.double() - r).abs().max() / r.abs().max())
+        worst = max(worst, err)
+        assert err < tol, f"request {n} position {p}: relative error {err:.2e}"
+    return worst
+
+
+def tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()

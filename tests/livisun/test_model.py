@@ -1,0 +1,121 @@
+"""Livisun through the engine (scheduler, paged cache, state slots, kernels or torch ops)
+against the slow oracle: whole prompts, decoding, portions, batches, reused pages and slots."""
+import pytest
+import torch
+
+from . import oracle
+from .common import SMALL, TAPS1, TAPS2, TAPS4, alone, build, check, run_schedule, tokens
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cfg", [SMALL, TAPS4, TAPS2, TAPS1], ids=["small", "taps4", "taps2", "taps1"])
+def test_whole_prompt_and_token_by_token(device, cfg):
+    eng, full = build(cfg, device)
+    t = tokens(75, cfg["vocab"], 1)
+    whole = run_schedule(eng, alone(t, []))
+    check(whole, cfg, full, {"a": t})
+    # the same tokens one at a time (every row a decode row), and a prompt then decoding
+    single = run_schedule(eng, alone(t, [1] * 74))
+    check(single, cfg, full, {"a": t})
+    mixed = run_schedule(eng, alone(t, [40] + [1] * 34))
+    check(mixed, cfg, full, {"a": t})
+    assert len(whole) == len(single) == len(mixed) == 75
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cuts", [[2] * 30, [3, 2, 33, 2, 5, 31, 2], [32, 32, 1, 1, 2], [64, 2],
+                                  [7, 7, 7, 7, 7, 7, 7, 7, 7, 7, 2, 1, 1]])
+def test_portions(device, cuts):
+    """Portions down to two tokens, cut inside pages and blocks; short ones run on the decode
+    kernel (<= 32 rows), long ones on the prefill kernel."""
+    eng, full = build(SMALL, device)
+    t = tokens(83, SMALL["vocab"], 2)
+    check(run_schedule(eng, alone(t, cuts)), SMALL, full, {"a": t})
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_first_tokens_and_one_token_requests(device):
+    eng, full = build(TAPS4, device)
+    for n in (1, 2, 3, 4):
+        t = tokens(n, TAPS4["vocab"], 10 + n)
+        check(run_schedule(eng, alone(t, [])), TAPS4, full, {"a": t})
+        check(run_schedule(eng, alone(t, [1] * n)), TAPS4, full, {"a": t})
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_batches_of_unequal_requests(device):
+    """Up to four live requests, portions beside single tokens, requests that pause, pages and
+    slots given back and used again by later requests: each row as if its request ran alone."""
+    cfg = SMALL
+    eng, full = build(cfg, device, max_kv_blocks=14)       # 13 pages: reuse is forced
+    V = cfg["vocab"]
+    req = {n: tokens(L, V, 20 + i) for i, (n, L) in enumerate(
+        [("a", 97), ("b", 40), ("c", 5), ("d", 66), ("e", 130), ("f", 33), ("g", 64)])}
+    at = {n: 0 for n in req}
+
+    def take(n, c):
+        lo = at[n]
+        at[n] = lo + c
+        return (n, req[n][lo:lo + c], list(range(c)))
+
+    plan = [
+        [("a", 50), ("b", 2), ("c", 5)], [("a", 1), ("b", 33), ("d", 40)], [("a", 1), ("b", 5)],
+        [("a", 45), ("d", 2)], [("d", 24), ("e", 64), ("f", 3)], [("e", 1), ("f", 30)],
+        [("e", 2), ("g", 64)], [("e", 63)],
+    ]
+    steps = []
+    for st in plan:
+        entries = [take(n, c) for n, c in st]
+        steps.append({"entries": entries, "end": [n for n, _ in st if at[n] == len(req[n])]})
+    assert all(at[n] == len(req[n]) for n in req)
+    got = run_schedule(eng, steps)
+    check(got, cfg, full, req)
+    assert len(got) == sum(len(t) for t in req.values())
+    assert eng.core.num_free_state_slots == 4 and eng.core.num_free_blocks == 13
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_slot_and_pages_reused_after_release(device):
+    """One slot, pool of one request: each request runs where the last one's state and keys
+    still lie."""
+    cfg = TAPS4
+    eng, full = build(cfg, device, max_num_seqs=1, max_kv_blocks=4)
+    for i in range(3):
+        t = tokens(70 + i, cfg["vocab"], 40 + i)
+        check(run_schedule(eng, alone(t, [33, 2, 1, 1])), cfg, full, {"a": t})
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decoding_over_block_and_page_edges(device):
+    cfg = TAPS2                                           # blocks of 33: edges off the pages
+    eng, full = build(cfg, device)
+    t = tokens(140, cfg["vocab"], 50)
+    check(run_schedule(eng, alone(t, [20] + [1] * 120)), cfg, full, {"a": t})
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_bfloat16_close_to_oracle(device):
+    eng, full = build(SMALL, device, dtype=torch.bfloat16)
+    t = tokens(60, SMALL["vocab"], 60)
+    got = run_schedule(eng, alone(t, [31, 2, 1, 1]))
+    ref = oracle.forward(SMALL, full, t)
+    for (_, p), row in got.items():
+        d = row.double() - ref[p]
+        d = d - d.mean()
+        assert float(d.pow(2).mean().sqrt() / ref.std()) < 0.08
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_through_the_engine(device):
+    """generate() (scheduler, sampler at temperature 0, decode steps) picks the oracle's tokens."""
+    from replisense_rfq_amd.engine.sequence import SamplingParams
+
+    cfg = SMALL
+    eng, full = build(cfg, device)
+    prompts = [tokens(n, cfg["vocab"], 70 + n) for n in (9, 35, 2)]
+    seqs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, grammar=False))
+    for p, s in zip(prompts, seqs):
+        assert s.output_ids == oracle.greedy(cfg, full, p, 12)
+    assert eng.core.num_free_state_slots == 4
