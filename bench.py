@@ -74,6 +74,10 @@ def parse():
     ap.add_argument("--kv-fraction", type=float, default=0.85,
                     help="fraction of free HBM for the paged KV pool (288 GB per MI355X)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--arch-compare", default="",
+                    help="livisun: instead of the RFQ workload, time prefill and decode of the "
+                         "layer-list model beside the Llama decoder at equal layer sizes "
+                         "(replisense_rfq_amd/benchmarks/arch_compare.py); one JSON line")
     ap.add_argument("--time-budget", type=float, default=0.0,
                     help="seconds; if > 0 the latency phase is skipped once this much wall "
                          "time has passed (the JSON line is always printed)")
@@ -358,6 +362,14 @@ def _any_rank(wctx, flag: bool) -> bool:
 def main():
     args = parse()
     t_start = time.perf_counter()
+    if args.arch_compare:
+        if args.arch_compare != "livisun" or args.gpus != 1:
+            raise SystemExit("bench: --arch-compare livisun runs on one GPU")
+        from replisense_rfq_amd.benchmarks import arch_compare
+
+        print(json.dumps({"metric": "arch_compare", "arch": args.arch_compare, "dtype": "bf16",
+                          "data": "synthetic", **arch_compare.run(args)}), flush=True)
+        return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(_self_launch(args))
 

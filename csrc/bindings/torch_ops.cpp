@@ -70,6 +70,9 @@ int prefill_split_tickets();
 void launch_sample_partial(const bf16_t*, int64_t, int, int, int, const uint32_t*, int,
                            const int32_t*, const float*, const uint64_t*, float*, int32_t*, int,
                            hipStream_t);
+void launch_sample_partial_f32(const float*, int64_t, int, int, int, const uint32_t*, int,
+                               const int32_t*, const float*, const uint64_t*, float*, int32_t*,
+                               int, hipStream_t);
 void launch_sample_final(const float*, const int32_t*, int, int, int, int32_t*, hipStream_t);
 void launch_moe_topk(const bf16_t*, int64_t, int, int, int, float*, int32_t*, bool, hipStream_t);
 void launch_moe_route(const bf16_t*, int64_t, const bf16_t*, int, int, int, int, float*, int32_t*,
@@ -630,7 +633,9 @@ std::vector<int64_t> prefill_split_ws_sizes() {
 void sample_partial(const Tensor& logits, int64_t v0, const Tensor& mask_table,
                     const Tensor& mask_idx, const Tensor& temps, const Tensor& seeds,
                     const Tensor& part_val, const Tensor& part_idx) {
-  CHECK_DEV(logits); CHECK_BF16(logits); CHECK_ROWMAJOR(logits);
+  CHECK_DEV(logits); CHECK_ROWMAJOR(logits);
+  const bool f32 = logits.scalar_type() == at::kFloat;
+  if (!f32) CHECK_BF16(logits);
   TORCH_CHECK(mask_table.scalar_type() == at::kInt && mask_table.dim() == 2 &&
                   mask_table.is_contiguous(),
               "mask_table must be int32 [n_masks, words]");
@@ -640,11 +645,22 @@ void sample_partial(const Tensor& logits, int64_t v0, const Tensor& mask_table,
   TORCH_CHECK(part_val.dim() == 2 && part_idx.dim() == 2, "partials must be [B, splits]");
   const int B = part_val.size(0), nsplit = part_val.size(1);
   const int Vl = logits.size(1);
-  TORCH_CHECK(Vl % 8 == 0 && v0 % 8 == 0, "vocab shard must be 8-aligned");
+  TORCH_CHECK((f32 || (Vl % 8 == 0 && logits.stride(0) % 8 == 0)) && v0 % 8 == 0,
+              "vocab shard must be 8-aligned");
   TORCH_CHECK(logits.size(0) >= B && mask_idx.numel() >= B && temps.numel() >= B &&
                   seeds.numel() >= B,
               "sample_partial: batch mismatch");
   TORCH_CHECK((v0 + Vl + 31) / 32 <= mask_table.size(1), "mask table too narrow");
+  if (f32) {
+    rfq::launch_sample_partial_f32(logits.data_ptr<float>(), logits.stride(0), B, Vl, v0,
+                                   reinterpret_cast<const uint32_t*>(mask_table.data_ptr<int32_t>()),
+                                   mask_table.size(1), mask_idx.data_ptr<int32_t>(),
+                                   temps.data_ptr<float>(),
+                                   reinterpret_cast<const uint64_t*>(seeds.data_ptr<int64_t>()),
+                                   part_val.data_ptr<float>(), part_idx.data_ptr<int32_t>(), nsplit,
+                                   cur_stream());
+    return;
+  }
   rfq::launch_sample_partial(bp(logits), logits.stride(0), B, Vl, v0,
                              reinterpret_cast<const uint32_t*>(mask_table.data_ptr<int32_t>()),
                              mask_table.size(1), mask_idx.data_ptr<int32_t>(),

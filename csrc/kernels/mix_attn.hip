@@ -283,6 +283,8 @@ __global__ __launch_bounds__(256) void attn_mixq_prefill_kernel(
 }
 
 // ------------------------------------------------------------------ launchers
+constexpr int kMaxLds = 160 * 1024;        // LDS of a gfx950 compute unit
+
 size_t decode_lds_floats(int H, int dim, int vdim, int KT) {
   return (size_t)H * dim + (size_t)KT * (dim + 1) + 2 * (size_t)H * KT + (size_t)H * H +
          (size_t)H * vdim + 3 * (size_t)H;
@@ -295,11 +297,24 @@ int launch_attn_talk_decode(bool f32, const float* qn, const void* k_cache, cons
                             int64_t out_stride, const float* slopes, const float* talk,
                             const float* sink, float scale, int chunk, int NA, int max_rows, int H,
                             int G, int dim, int vdim, int BS, hipStream_t s) {
+  // the largest key tile whose LDS fits two workgroups per CU, else one (160 KB per CU)
   int KT = 64;
-  while (KT >= 8 && decode_lds_floats(H, dim, vdim, KT) * 4 > 64 * 1024) KT >>= 1;
+  while (KT >= 8 && decode_lds_floats(H, dim, vdim, KT) * 4 > 80 * 1024) KT >>= 1;
+  if (KT < 8) {
+    KT = 64;
+    while (KT >= 8 && decode_lds_floats(H, dim, vdim, KT) * 4 > kMaxLds) KT >>= 1;
+  }
   if (KT < 8) return 0;
   if (NA == 0) return KT;
   const size_t lds = decode_lds_floats(H, dim, vdim, KT) * 4;
+  static bool attr = false;
+  if (!attr) {          // dynamic LDS above 64 KB has to be allowed per kernel, once
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_talk_decode_kernel<float>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_talk_decode_kernel<bf16_t>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    attr = true;
+  }
   if (f32)
     hipLaunchKernelGGL(attn_talk_decode_kernel<float>, dim3(NA, max_rows), dim3(256), lds, s, qn,
                        (const float*)k_cache, (const float*)v_cache, bt, maxb, q_start, q_len,
@@ -321,8 +336,16 @@ bool launch_attn_mixq_prefill(bool f32, const float* qmix, const void* k_cache,
                               int H, int G, int dim, int vdim, int BS, hipStream_t s) {
   const size_t lds = ((size_t)QB * (EC + 1) + (size_t)KT2 * (EC + 1) + (size_t)QB * (KT2 + 1) +
                       (size_t)QB * vdim + 2 * QB) * 4;
-  if (lds > 64 * 1024) return false;
+  if (lds > (size_t)kMaxLds) return false;
   if (W == 0) return true;
+  static bool attr = false;
+  if (!attr) {
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mixq_prefill_kernel<float>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mixq_prefill_kernel<bf16_t>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    attr = true;
+  }
   if (f32)
     hipLaunchKernelGGL(attn_mixq_prefill_kernel<float>, dim3(W, H), dim3(256), lds, s, qmix,
                        (const float*)k_cache, (const float*)v_cache, bt, maxb, q_start, q_len,

@@ -208,7 +208,7 @@ void launch_head_norm_append(bool f32, const void* qkv, int64_t stride, const fl
                              void* v_cache, int T_, int H, int G, int dim, int vdim, int BS,
                              float* qn, const float* ts, float* qmix, int mix_from, hipStream_t s) {
   if (T_ == 0) return;
-  const size_t lds = (size_t)H * dim * sizeof(float);
+  const size_t lds = (size_t)H * dim * sizeof(float);       // checked <= 64 KB by the caller
   MIX_DISPATCH(f32, hipLaunchKernelGGL(head_norm_append_kernel<T>, dim3(T_), dim3(256), lds, s,
                                        (const T*)qkv, stride, q_w, k_w, eps, slots, (T*)k_cache,
                                        (T*)v_cache, H, G, dim, vdim, BS, qn, ts, qmix, mix_from));

@@ -17,8 +17,19 @@ namespace rfq {
 
 constexpr int kSampleBlock = 256;
 
+// 8 logits from column c of a row: one 16-byte load of bf16 (Vl and the row stride are
+// multiples of 8 then), or guarded scalar loads of fp32 logits (any Vl).
+__device__ __forceinline__ void load8(const bf16_t* row, int c, int c1, float* f) {
+  unpack8(reinterpret_cast<const s16x8*>(row + c)[0], f);
+}
+__device__ __forceinline__ void load8(const float* row, int c, int c1, float* f) {
+#pragma unroll
+  for (int k = 0; k < 8; ++k) f[k] = c + k < c1 ? row[c + k] : 0.f;
+}
+
+template <typename LT>
 __global__ __launch_bounds__(kSampleBlock) void sample_partial_kernel(
-    const bf16_t* __restrict__ logits, int64_t row_stride, int Vl, int v0,
+    const LT* __restrict__ logits, int64_t row_stride, int Vl, int v0,
     const uint32_t* __restrict__ mask_table, int mask_words, const int32_t* __restrict__ mask_idx,
     const float* __restrict__ temps, const uint64_t* __restrict__ seeds,
     float* __restrict__ part_val, int32_t* __restrict__ part_idx, int chunk) {
@@ -31,7 +42,7 @@ __global__ __launch_bounds__(kSampleBlock) void sample_partial_kernel(
   const float t = temps[b];
   const float invT = t > 0.f ? 1.f / t : 0.f;
   const uint64_t seed = seeds[b];
-  const bf16_t* row = logits + (int64_t)b * row_stride;
+  const LT* row = logits + (int64_t)b * row_stride;
 
   float best = -INFINITY;
   int besti = 0x7fffffff;
@@ -40,11 +51,12 @@ __global__ __launch_bounds__(kSampleBlock) void sample_partial_kernel(
     uint32_t bits = 0xffu;
     if (mrow) bits = (mrow[gcol >> 5] >> (gcol & 31)) & 0xffu;
     if (bits == 0) continue;
-    const s16x8 v = reinterpret_cast<const s16x8*>(row + c)[0];
+    float v[8];
+    load8(row, c, c1, v);
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       if (!((bits >> k) & 1u) || c + k >= c1) continue;
-      float sc = bf2f_s(v[k]);
+      float sc = v[k];
       if (t > 0.f) {
         const uint32_t hsh = hash_u32(seed, 0x9e3779b9u, (uint32_t)(gcol + k));
         const float u = ((float)(hsh >> 8) + 0.5f) * (1.f / 16777216.f);
@@ -100,17 +112,36 @@ __global__ __launch_bounds__(64) void sample_final_kernel(const float* __restric
   if (threadIdx.x == 0) out_tokens[b] = besti == 0x7fffffff ? 0 : besti;
 }
 
-void launch_sample_partial(const bf16_t* logits, int64_t row_stride, int B, int Vl, int v0,
-                           const uint32_t* mask_table, int mask_words, const int32_t* mask_idx,
-                           const float* temps, const uint64_t* seeds, float* part_val,
-                           int32_t* part_idx, int nsplit, hipStream_t s) {
+template <typename LT>
+static void sample_partial_launch(const LT* logits, int64_t row_stride, int B, int Vl, int v0,
+                                  const uint32_t* mask_table, int mask_words,
+                                  const int32_t* mask_idx, const float* temps,
+                                  const uint64_t* seeds, float* part_val, int32_t* part_idx,
+                                  int nsplit, hipStream_t s) {
   if (B == 0) return;
   int chunk = (Vl + nsplit - 1) / nsplit;
   chunk = (chunk + 7) / 8 * 8;
   dim3 grid(nsplit, B);
-  sample_partial_kernel<<<grid, kSampleBlock, 0, s>>>(logits, row_stride, Vl, v0, mask_table,
-                                                      mask_words, mask_idx, temps, seeds,
-                                                      part_val, part_idx, chunk);
+  sample_partial_kernel<LT><<<grid, kSampleBlock, 0, s>>>(logits, row_stride, Vl, v0, mask_table,
+                                                          mask_words, mask_idx, temps, seeds,
+                                                          part_val, part_idx, chunk);
+}
+
+void launch_sample_partial(const bf16_t* logits, int64_t row_stride, int B, int Vl, int v0,
+                           const uint32_t* mask_table, int mask_words, const int32_t* mask_idx,
+                           const float* temps, const uint64_t* seeds, float* part_val,
+                           int32_t* part_idx, int nsplit, hipStream_t s) {
+  sample_partial_launch(logits, row_stride, B, Vl, v0, mask_table, mask_words, mask_idx, temps,
+                        seeds, part_val, part_idx, nsplit, s);
+}
+
+// fp32 logits (models whose head keeps the accumulator's precision); any vocabulary size
+void launch_sample_partial_f32(const float* logits, int64_t row_stride, int B, int Vl, int v0,
+                               const uint32_t* mask_table, int mask_words,
+                               const int32_t* mask_idx, const float* temps, const uint64_t* seeds,
+                               float* part_val, int32_t* part_idx, int nsplit, hipStream_t s) {
+  sample_partial_launch(logits, row_stride, B, Vl, v0, mask_table, mask_words, mask_idx, temps,
+                        seeds, part_val, part_idx, nsplit, s);
 }
 
 void launch_sample_final(const float* part_val, const int32_t* part_idx, int B, int n,

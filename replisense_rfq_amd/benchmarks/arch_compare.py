@@ -1,0 +1,94 @@
+"""Prefill and decode throughput of a layer-list model beside the Llama decoder at equal
+layer sizes (``bench.py --arch-compare livisun``).
+
+Both run through the same engine (scheduler, paged cache, hipGraph decode steps), with
+random weights, a few layers of a real model's shape and a small vocabulary, so the numbers
+compare the layers' kernels:
+
+  prefill  P prompts of S tokens in steps of at most --prefill-chunk tokens  -> tokens/s
+  decode   B sequences, N sampled tokens each (temperature 0)                -> tokens/s
+"""
+from __future__ import annotations
+
+import time
+
+import torch
+
+from ..engine.engine import LLMEngine
+from ..engine.sequence import SamplingParams
+from ..models.config import LayeredConfig, LayerSpec, MixerSpec, MlpSpec, ModelConfig
+from ..utils.config import EngineConfig
+
+# (name, hidden, q heads, kv heads, ff) with 128-wide heads (the Llama kernels' head size)
+SIZES = [("1b-class", 2048, 16, 4, 8192), ("8b-class", 4096, 32, 8, 14336),
+         ("70b-class", 8192, 64, 8, 28672)]
+LAYERS, VOCAB, CHUNK = 4, 32000, 2048
+
+
+def _configs(name, d, H, G, F):
+    llama = ModelConfig(f"cmp-llama-{name}", vocab_size=VOCAB, hidden=d, n_layers=LAYERS,
+                        n_heads=H, n_kv_heads=G, ffn=F, bos_id=1, eos_ids=())
+    mix = MixerSpec("attention", H, G, 128, 128, 128 ** -0.5, CHUNK)
+    liv = LayeredConfig(f"cmp-livisun-{name}", vocab_size=VOCAB, hidden=d,
+                        layers=tuple(LayerSpec(mix, MlpSpec("dense", F, 7.0)) for _ in range(LAYERS)))
+    return llama, liv
+
+
+def _engine(mcfg, args, batch):
+    from ..models.livisun import LivisunLM
+    from ..models.llama import DecoderLM
+
+    dev = torch.device("cuda", 0)
+    model = (LivisunLM if isinstance(mcfg, LayeredConfig) else DecoderLM)(mcfg, dev, seed=args.seed)
+    cfg = EngineConfig(model=mcfg.name, max_num_seqs=batch, max_kv_blocks=batch * 80 + 64,
+                       max_batched_tokens=args.prefill_chunk, max_model_len=2560,
+                       use_graphs=not args.no_graphs, graph_buckets=(batch,), grammar=False,
+                       prefix_cache=False, warm_prefix=False, jump_forward=False,
+                       tune_gemm=not isinstance(mcfg, LayeredConfig))
+    return LLMEngine(cfg, model=model)
+
+
+def _measure(eng, prompts, new_tokens):
+    """(prefill tokens/s, decode tokens/s): the prompts' steps, then the decode steps."""
+    sp = SamplingParams(temperature=0.0, max_tokens=new_tokens, grammar=False)
+    for p in prompts:
+        eng.add_request(p, sp)
+    n_prompt = sum(len(p) for p in prompts)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while eng.has_work() and eng.core.num_waiting + sum(
+            1 for s in eng._live.values() if eng.core.info(s.core_id)["num_cached"] < len(s.prompt)):
+        eng.step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    steps = 0
+    while eng.has_work():
+        eng.step()
+        steps += 1
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    return n_prompt / (t1 - t0), steps * len(prompts) / (t2 - t1), steps
+
+
+def run(args) -> dict:
+    g = torch.Generator().manual_seed(args.seed)
+    out = {"layers": LAYERS, "vocab": VOCAB, "block": CHUNK, "prompt": [8, 2048],
+           "decode": [64, 128], "sizes": {}}
+    for name, d, H, G, F in SIZES:
+        row = {}
+        for mcfg in _configs(name, d, H, G, F):
+            kind = "livisun" if isinstance(mcfg, LayeredConfig) else "llama"
+            eng = _engine(mcfg, args, 64)
+            pre = [torch.randint(2, VOCAB, (2048,), generator=g).tolist() for _ in range(8)]
+            dec = [torch.randint(2, VOCAB, (512,), generator=g).tolist() for _ in range(64)]
+            _measure(eng, pre[:2], 2)                              # warm-up
+            p_tps, _, _ = _measure(eng, pre, 1)
+            _, d_tps, steps = _measure(eng, dec, 128)
+            row[kind] = {"prefill_tok_s": round(p_tps), "decode_tok_s": round(d_tps),
+                         "decode_steps": steps, "graph_steps": eng.runner.stats["graph_steps"]}
+            del eng
+            torch.cuda.empty_cache()
+        row["prefill_ratio"] = round(row["livisun"]["prefill_tok_s"] / row["llama"]["prefill_tok_s"], 3)
+        row["decode_ratio"] = round(row["livisun"]["decode_tok_s"] / row["llama"]["decode_tok_s"], 3)
+        out["sizes"][name] = row
+    return out

@@ -1004,6 +1004,9 @@ def reset_plans() -> None:
 # Ops of the layer-list models (csrc/kernels/mix_*.hip, library _C_mix.so).  The
 # residual stream and every norm are fp32; activations that feed matrix products
 # have the model's dtype (bf16, or fp32 for a model served in full precision).
+_MM_OUT_DTYPE = None      # whether torch.mm takes out_dtype on this build (probed once)
+
+
 def matmul_nt(x, w, out_dtype=None):
     """x[M, K] . w[N, K]^T on the vendor library (fp32 accumulation; true fp32 for fp32
     operands); ``out_dtype`` float32 keeps the accumulator's precision for bf16 operands."""
@@ -1011,11 +1014,16 @@ def matmul_nt(x, w, out_dtype=None):
         return x @ w.t()
     if x.shape[0] == 0:
         return torch.empty((0, w.shape[0]), dtype=out_dtype, device=x.device)
-    if x.is_cuda:
-        try:
+    global _MM_OUT_DTYPE
+    if x.is_cuda and _MM_OUT_DTYPE is not False:
+        if _MM_OUT_DTYPE:
             return torch.mm(x, w.t(), out_dtype=out_dtype)
+        try:                                   # first call (never inside a graph capture)
+            y = torch.mm(x, w.t(), out_dtype=out_dtype)
+            _MM_OUT_DTYPE = True
+            return y
         except (TypeError, RuntimeError):
-            pass
+            _MM_OUT_DTYPE = False
     return x.to(out_dtype) @ w.to(out_dtype).t()
 
 

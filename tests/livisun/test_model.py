@@ -6,7 +6,7 @@ import torch
 from . import oracle
 from .common import SMALL, TAPS1, TAPS2, TAPS4, alone, build, check, run_schedule, tokens
 
-DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
 
 
 @pytest.mark.parametrize("device", DEVICES)
