@@ -33,6 +33,7 @@ bool launch_attn_mixq_prefill_mfma(const float*, const void*, const void*, const
                                    const int32_t*, const int32_t*, const int32_t*, const int32_t*,
                                    const int32_t*, int, void*, int64_t, const float*, const float*,
                                    int, int, int, int, int, int, hipStream_t);
+bool mixq_mfma_ok(int, int, int, int, int);
 }  // namespace rfqmix
 
 namespace {
@@ -211,6 +212,10 @@ void attn_mixq_prefill(const Tensor& qmix, const Tensor& k_cache, const Tensor& 
   TORCH_CHECK(ok, "attn_mixq_prefill: value size does not fit the LDS");
 }
 
+bool mixq_mfma_ok(int64_t H, int64_t G, int64_t dim, int64_t vdim, int64_t BS) {
+  return rfqmix::mixq_mfma_ok((int)H, (int)G, (int)dim, (int)vdim, (int)BS);
+}
+
 void glu_clamped(const Tensor& gu, double limit, double alpha, const Tensor& out) {
   const bool f32 = act_f32(gu, "glu_clamped gate_up");
   const int T = (int)gu.size(0), F = (int)out.size(1);
@@ -232,6 +237,7 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("attn_talk_decode(Tensor qn, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor(a!) out, Tensor slopes, Tensor? talk, Tensor? sink, float scale, int chunk, int max_rows) -> ()");
   m.def("attn_mixq_prefill(Tensor qmix, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor slopes, Tensor? sink, int chunk, int qblk, int mfma) -> ()");
   m.def("glu_clamped(Tensor gate_up, float limit, float alpha, Tensor(a!) out) -> ()");
+  m.def("mixq_mfma_ok", &mixq_mfma_ok);
 }
 
 TORCH_LIBRARY_IMPL(rfq_mix, CUDA, m) {

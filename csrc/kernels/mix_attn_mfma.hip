@@ -1,12 +1,222 @@
-// MFMA form of attn_mixq_prefill for bf16 models (see mix_attn.hip for the math).
-#include "mix_common.h"
+// MFMA form of attn_mixq_prefill for bf16 models (the math is at the top of mix_attn.hip).
+//
+// Queries arrive mixed and scaled, [T, H, E] with E = G * dim, so the mixed score of head h
+// is ONE product with the concatenation of all G key heads, and every head of a token reads
+// the same keys.  A work item is (sequence, block of 32 query tokens, key/value head c); its
+// columns are the (token, head) pairs of the heads that use value head c, 16 per wave:
+//
+//   S^T[key, col]  = K_cat[key, :] . Q~[col, :]         v_mfma_f32_16x16x32_bf16, A = keys
+//   bias, block mask, online softmax per column (fp32; the sink is the initial state)
+//   O^T[dv, col]  += V_c^T[dv, key] . P^T[key, col]      A = V^T by transposed LDS reads,
+//                                                        P split into bf16 hi + lo parts so
+//                                                        the weights keep fp32's precision
+//
+// One key tile is one 32-token page.  The waves of a workgroup share the page's V tile in
+// LDS; K fragments go straight from the cache to registers (16 B per lane).  The same kernel
+// serves the decode section (one token x rep heads per column tile).
+#include "common.h"
 
 namespace rfqmix {
 
-bool launch_attn_mixq_prefill_mfma(const float*, const void*, const void*, const int32_t*, int,
-                                   const int32_t*, const int32_t*, const int32_t*, const int32_t*,
-                                   const int32_t*, int, void*, int64_t, const float*, const float*,
-                                   int, int, int, int, int, int, hipStream_t) {
+using namespace rfq;
+
+constexpr int kPg = 32;
+
+template <int EK, int VT>
+__global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
+    const float* __restrict__ qmix, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int maxb,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
+    const int32_t* __restrict__ kv_len, const int32_t* __restrict__ work_seq,
+    const int32_t* __restrict__ work_qblk, bf16_t* __restrict__ out, int64_t out_stride,
+    const float* __restrict__ slopes, const float* __restrict__ sink, int chunk, int H, int G,
+    int dim) {
+  constexpr int VD = VT * 16, E = EK * 32;
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[kPg * VD];
+  const int s = work_seq[blockIdx.x];
+  if (s < 0) return;
+  const int ql = q_len[s], kl = kv_len[s];
+  const int i0 = work_qblk[blockIdx.x] * 32;
+  if (i0 >= ql) return;
+  const int nq = min(32, ql - i0);
+  const int cg = blockIdx.y, rep = H / G;
+  const int nwaves = blockDim.x >> 6, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int g4 = lane >> 4, c = lane & 15;
+  const int tile = blockIdx.z * nwaves + wave;
+  const bool active = tile * 16 < nq * rep;             // wave-uniform
+  const int col = tile * 16 + c;
+  const int tok = col / rep, hh = cg * rep + col % rep;
+  const bool cvalid = active && tok < nq;
+  const int p0 = kl - ql + i0, plast = p0 + nq - 1;
+  const int pi = p0 + (cvalid ? tok : 0);
+  const int ci = chunk > 0 ? pi / chunk : 0;
+  const int jlo = chunk > 0 ? (p0 / chunk) * chunk : 0;
+  const int32_t* bt = block_tables + (int64_t)s * maxb;
+  const float slope = slopes[hh < H ? hh : 0];
+
+  // mixed queries of this lane's column as B operands (k = 8 g4 + j of every 32-slice)
+  s16x8 qf[EK];
+  {
+    const float* qr = qmix + ((int64_t)(q_start[s] + i0 + (cvalid ? tok : 0)) * H + (cvalid ? hh : 0)) * E;
+#pragma unroll
+    for (int ks = 0; ks < EK; ++ks) {
+      float f[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = cvalid ? qr[32 * ks + 8 * g4 + j] : 0.f;
+      qf[ks] = pack8(f);
+    }
+  }
+  // element offset of every 32-slice of the concatenated key inside a page (wave-uniform)
+  int koff[EK];
+#pragma unroll
+  for (int ks = 0; ks < EK; ++ks) {
+    const int ck = (32 * ks) / dim;
+    koff[ks] = ck * kPg * dim + (32 * ks - ck * dim);
+  }
+  const int klane = c * dim + 8 * g4;
+  f32x4 o[VT];
+#pragma unroll
+  for (int m = 0; m < VT; ++m) o[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m_run = (sink != nullptr && cvalid) ? sink[hh] : -INFINITY;
+  float l_run = (sink != nullptr && cvalid) ? 1.f : 0.f;
+
+  for (int pg = jlo / kPg; pg <= plast / kPg; ++pg) {
+    const int kt = pg * kPg;
+    const int64_t page = bt[pg];
+    // V tile of value head cg -> LDS; rows past the last written key are zeroed (they may
+    // hold anything, and 0 * NaN would poison the sum)
+    {
+      const bf16_t* vb = v_cache + ((page * G + cg) * kPg) * (int64_t)VD;
+      for (int x = threadIdx.x; x < kPg * VD / 8; x += blockDim.x) {
+        const int row = x / (VD / 8);
+        s16x8 v = reinterpret_cast<const s16x8*>(vb)[x];
+        if (kt + row > plast) v = (s16x8){0, 0, 0, 0, 0, 0, 0, 0};
+        reinterpret_cast<s16x8*>(v_lds)[x] = v;
+      }
+    }
+    s16x8 pb_hi = (s16x8){0, 0, 0, 0, 0, 0, 0, 0}, pb_lo = pb_hi;
+    float alpha = 1.f;
+    if (active) {
+      f32x4 sc[2];
+      const bf16_t* kp = k_cache + page * G * kPg * (int64_t)dim + klane;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        sc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < EK; ++ks) {
+          const s16x8 kf = *reinterpret_cast<const s16x8*>(kp + koff[ks] + 16 * mt * dim);
+          sc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[ks]),
+                                                           sc[mt], 0, 0, 0);
+        }
+      }
+      // lane holds S^T[key = kt + 16 mt + 4 g4 + i][column c]
+      float mx = -INFINITY;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kt + 16 * mt + 4 * g4 + i;
+          const bool ok = cvalid && key <= pi && (chunk == 0 || key / chunk == ci);
+          const float v = ok ? sc[mt][i] - slope * (float)(pi - key) : -INFINITY;
+          sc[mt][i] = v;
+          mx = fmaxf(mx, v);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      alpha = __expf(m_run - m_use);
+      float psum = 0.f, ph[8], pl[8];
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const float p = __expf(sc[jj >> 2][jj & 3] - m_use);
+        psum += p;
+        ph[jj] = bf2f(f2bf(p));
+        pl[jj] = p - ph[jj];
+      }
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+      l_run = l_run * alpha + psum;
+      m_run = m_new;
+      // P^T as B operand: element j <-> key (j < 4 ? 4 g4 + j : 16 + 4 g4 + j - 4)
+      pb_hi = pack8(ph);
+      pb_lo = pack8(pl);
+    }
+    __syncthreads();                                   // V tile visible
+    if (active) {
+      const int q4 = c >> 2, p4 = c & 3;
+#pragma unroll
+      for (int m = 0; m < VT; ++m) {
+        const int r0 = 4 * g4 + q4, r1 = 16 + 4 * g4 + q4;
+        const s16x4 a0 = ds_read_tr16(v_lds + r0 * VD + 16 * m + 4 * p4);
+        const s16x4 a1 = ds_read_tr16(v_lds + r1 * VD + 16 * m + 4 * p4);
+        const s16x8 a = (s16x8){a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+        o[m] *= alpha;
+        o[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(pb_hi), o[m], 0, 0, 0);
+        o[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(pb_lo), o[m], 0, 0, 0);
+      }
+    }
+    __syncthreads();                                   // before the next page overwrites it
+  }
+  if (!cvalid) return;
+  // lane holds O^T[dv = 16 m + 4 g4 + i][column c]
+  const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+  bf16_t* orow = out + (int64_t)(q_start[s] + i0 + tok) * out_stride + (int64_t)hh * VD;
+#pragma unroll
+  for (int m = 0; m < VT; ++m) {
+    uint2 w;
+    w.x = pack_bf16x2(o[m][0] * inv, o[m][1] * inv);
+    w.y = pack_bf16x2(o[m][2] * inv, o[m][3] * inv);
+    *reinterpret_cast<uint2*>(orow + 16 * m + 4 * g4) = w;
+  }
+}
+
+template <int EK, int VT>
+static void launch_one(const float* qmix, const bf16_t* k, const bf16_t* v, const int32_t* bt,
+                       int maxb, const int32_t* q_start, const int32_t* q_len,
+                       const int32_t* kv_len, const int32_t* work_seq, const int32_t* work_qblk,
+                       int W, bf16_t* out, int64_t out_stride, const float* slopes,
+                       const float* sink, int chunk, int H, int G, int dim, hipStream_t s) {
+  const int rep = H / G;
+  const int nwaves = 2 * rep < 4 ? 2 * rep : 4;
+  const int z = (2 * rep + nwaves - 1) / nwaves;
+  hipLaunchKernelGGL((attn_mixq_mfma_kernel<EK, VT>), dim3(W, G, z), dim3(nwaves * 64), 0, s, qmix,
+                     k, v, bt, maxb, q_start, q_len, kv_len, work_seq, work_qblk, out, out_stride,
+                     slopes, sink, chunk, H, G, dim);
+}
+
+// Sizes the MFMA tiles cover: 32-token pages, dim a multiple of 32, E = G dim in
+// {64, 128, 256, 512, 1024}, vdim in {32, 64, 128}, 16 a multiple of the heads per value head.
+bool mixq_mfma_ok(int H, int G, int dim, int vdim, int BS) {
+  const int rep = G > 0 ? H / G : 0, E = G * dim;
+  return BS == kPg && rep >= 1 && H == rep * G && 16 % rep == 0 && dim % 32 == 0 &&
+         (E == 64 || E == 128 || E == 256 || E == 512 || E == 1024) &&
+         (vdim == 32 || vdim == 64 || vdim == 128) && G <= 65535;
+}
+
+bool launch_attn_mixq_prefill_mfma(const float* qmix, const void* k_cache, const void* v_cache,
+                                   const int32_t* bt, int maxb, const int32_t* q_start,
+                                   const int32_t* q_len, const int32_t* kv_len,
+                                   const int32_t* work_seq, const int32_t* work_qblk, int W,
+                                   void* out, int64_t out_stride, const float* slopes,
+                                   const float* sink, int chunk, int H, int G, int dim, int vdim,
+                                   int BS, hipStream_t s) {
+  if (!mixq_mfma_ok(H, G, dim, vdim, BS)) return false;
+  if (W == 0) return true;
+  const int EK = G * dim / 32, VT = vdim / 16;
+#define MIXQ_CASE(ek, vt)                                                                       \
+  if (EK == ek && VT == vt) {                                                                   \
+    launch_one<ek, vt>(qmix, (const bf16_t*)k_cache, (const bf16_t*)v_cache, bt, maxb, q_start, \
+                       q_len, kv_len, work_seq, work_qblk, W, (bf16_t*)out, out_stride, slopes, \
+                       sink, chunk, H, G, dim, s);                                              \
+    return true;                                                                                \
+  }
+  MIXQ_CASE(2, 2) MIXQ_CASE(2, 4) MIXQ_CASE(2, 8)
+  MIXQ_CASE(4, 2) MIXQ_CASE(4, 4) MIXQ_CASE(4, 8)
+  MIXQ_CASE(8, 2) MIXQ_CASE(8, 4) MIXQ_CASE(8, 8)
+  MIXQ_CASE(16, 2) MIXQ_CASE(16, 4) MIXQ_CASE(16, 8)
+  MIXQ_CASE(32, 2) MIXQ_CASE(32, 4) MIXQ_CASE(32, 8)
+#undef MIXQ_CASE
   return false;
 }
 

@@ -73,6 +73,11 @@ class LivisunLM:
             lw["slopes"] = slopes
             lw["talk_scaled"] = (lw["talk"] * m.scale).contiguous()
             lw["slopes_mixed"] = (lw["talk"].double() @ slopes.double()).float().contiguous()
+            # bf16 on the GPU with sizes the MFMA tiles cover: decode rows too run the
+            # mixed-query kernel (one work item per sequence); otherwise attn_talk_decode
+            lw["mixq_decode"] = bool(self.device.type == "cuda" and dtype == torch.bfloat16
+                                     and ops.mixq_mfma_ok(m.heads, m.kv_heads, m.dim, m.vdim))
+        self._seq_ids = None            # work list of the decode section: sequence j, block 0
 
     # engine hooks shared with DecoderLM
     def fold_norms(self) -> bool:
@@ -85,6 +90,15 @@ class LivisunLM:
         """Per-layer pools [num_blocks, G, block, dim | vdim]; state [L, 2, 2*slots, taps-1, d]."""
         assert len(k_pools) == self.cfg.n_layers
         self.kv_k, self.kv_v, self.state = k_pools, v_pools, state
+
+    def _decode_work(self, n: int):
+        """(sequence index, query block 0) per decode-section sequence; views of two
+        tensors that only grow (never inside a graph capture: the warm-up run sizes them)."""
+        if self._seq_ids is None or self._seq_ids[0].numel() < n:
+            size = max(1024, 2 * n)
+            self._seq_ids = (torch.arange(size, dtype=torch.int32, device=self.device),
+                             torch.zeros(size, dtype=torch.int32, device=self.device))
+        return self._seq_ids[0][:n], self._seq_ids[1][:n]
 
     def weight_bytes(self) -> int:
         tot = sum(v.numel() * v.element_size() for v in self.w.values() if isinstance(v, torch.Tensor))
@@ -112,17 +126,25 @@ class LivisunLM:
             ops.canon_conv(h, lw["canon1"], self.state[li, 0], rs, rb, rf, pos, hc)
             qkv = ops.matmul_nt(hc, lw["qkv"])
             qn = torch.empty((T, H, dim), dtype=torch.float32, device=dev)
-            qmix = torch.empty((T - D, H, G * dim), dtype=torch.float32, device=dev) if T > D else None
+            mix_from = 0 if lw["mixq_decode"] else D
+            qmix = torch.empty((T - mix_from, H, G * dim), dtype=torch.float32, device=dev) \
+                if T > mix_from else None
             ops.head_norm_append(qkv, lw["q_norm"], lw["k_norm"], eps, m.slot_mapping[:T],
                                  self.kv_k[li], self.kv_v[li], H, G, dim, vd, qn,
-                                 lw["talk_scaled"], qmix, D)
+                                 lw["talk_scaled"], qmix, mix_from)
             attn = torch.empty((T, H * vd), dtype=dt, device=dev)
-            if D > 0:
+            if D > 0 and lw["mixq_decode"]:
+                NA = m.dec_q_len.shape[0]
+                ids, zeros = self._decode_work(NA)
+                ops.attn_mixq_prefill(qmix[:D], self.kv_k[li], self.kv_v[li], m.dec_block_tables,
+                                      m.dec_q_start, m.dec_q_len, m.dec_kv_len, ids, zeros,
+                                      attn[:D], lw["slopes_mixed"], lw["sink"], mx.chunk)
+            elif D > 0:
                 ops.attn_talk_decode(qn[:D], self.kv_k[li], self.kv_v[li], m.dec_block_tables,
                                      m.dec_q_start, m.dec_q_len, m.dec_kv_len, attn[:D],
                                      lw["slopes"], lw["talk"], lw["sink"], mx.scale, mx.chunk)
             if T > D:
-                ops.attn_mixq_prefill(qmix, self.kv_k[li], self.kv_v[li], m.pf_block_tables,
+                ops.attn_mixq_prefill(qmix[D - mix_from:], self.kv_k[li], self.kv_v[li], m.pf_block_tables,
                                       m.pf_q_start, m.pf_q_len, m.pf_kv_len, m.work_seq,
                                       m.work_qblk, attn[D:T], lw["slopes_mixed"], lw["sink"],
                                       mx.chunk, m.prefill_qblk)

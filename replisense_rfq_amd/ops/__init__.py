@@ -1102,6 +1102,11 @@ def attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len, kv_l
                               slopes, sink, chunk)
 
 
+def mixq_mfma_ok(H: int, G: int, dim: int, vdim: int, block: int = 32) -> bool:
+    """Whether the MFMA tiles of attn_mixq_prefill cover these sizes (bf16 caches, GPU)."""
+    return bool(MIXQ_MFMA and _native.mix_ops().mixq_mfma_ok(H, G, dim, vdim, block))
+
+
 def glu_clamped(gate_up, limit: float, alpha: float = 1.702, out=None):
     F = gate_up.shape[1] // 2
     out = torch.empty((gate_up.shape[0], F), dtype=gate_up.dtype, device=gate_up.device) \

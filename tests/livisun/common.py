@@ -28,6 +28,9 @@ SMALL = config([layer(6, 2, 16, 8, 7, 40), layer(2, 1, 24, 24, 20, None), layer(
 TAPS4 = config([layer(4, 2, 8, 8, 11, 32, scale=0.5, limit=0.7), layer(4, 4, 16, 8, 64, 16)],
                width=40, taps=4, emb=1.0)
 TAPS2 = config([layer(2, 2, 32, 16, 33, 56)], width=64, taps=2, emb=7.0, eps=1e-3)
+# sizes the MFMA attention tiles cover (bf16 on the GPU): wide keys, 4 and 1 heads per value head
+WIDE = config([layer(8, 2, 32, 32, 40, 64, scale=0.2), layer(4, 4, 64, 64, 0, 64, scale=0.15),
+               layer(4, 2, 32, 64, 33, None, scale=0.2)], width=64, vocab=90)
 TAPS1 = config([layer(4, 1, 16, 16, 5, 24)], width=32, taps=1)
 
 

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from . import oracle
-from .common import SMALL, TAPS1, TAPS2, TAPS4, alone, build, check, run_schedule, tokens
+from .common import SMALL, TAPS1, TAPS2, TAPS4, WIDE, alone, build, check, run_schedule, tokens
 
 DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
 
@@ -105,6 +105,33 @@ def test_bfloat16_close_to_oracle(device):
         d = row.double() - ref[p]
         d = d - d.mean()
         assert float(d.pow(2).mean().sqrt() / ref.std()) < 0.08
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_wide_heads_in_batches(device, dtype):
+    """Head sizes of the matrix-core attention tiles: portions, single tokens and a batch; in
+    bf16 every row stays within rounding of the oracle and does not depend on the cut."""
+    cfg = WIDE
+    eng, full = build(cfg, device, dtype=dtype)
+    a, b = tokens(100, cfg["vocab"], 80), tokens(41, cfg["vocab"], 81)
+    steps = [{"entries": [("a", a[:70], list(range(70))), ("b", b[:3], [0, 1, 2])], "end": []},
+             {"entries": [("a", a[70:71], [0]), ("b", b[3:40], list(range(37)))], "end": []},
+             {"entries": [("a", a[71:], list(range(29))), ("b", b[40:], [0])], "end": ["a", "b"]}]
+    got = run_schedule(eng, steps)
+    assert len(got) == 141
+    if dtype == torch.float32:
+        check(got, cfg, full, {"a": a, "b": b})
+        return
+    ref = {"a": oracle.forward(cfg, full, a), "b": oracle.forward(cfg, full, b)}
+    for (n, p), row in got.items():
+        d = row.double() - ref[n][p]
+        d = d - d.mean()
+        assert float(d.pow(2).mean().sqrt() / ref[n].std()) < 0.08, (n, p)
+    whole = run_schedule(eng, alone(a, []))
+    for p in range(100):
+        d = (whole[("a", p)] - got[("a", p)]).double()
+        assert float(d.pow(2).mean().sqrt() / ref["a"].std()) < 0.08
 
 
 @pytest.mark.parametrize("device", DEVICES)
