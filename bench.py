@@ -74,6 +74,7 @@ def parse():
     ap.add_argument("--kv-fraction", type=float, default=0.85,
                     help="fraction of free HBM for the paged KV pool (288 GB per MI355X)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--arch-sizes", default="", help="--arch-compare: size classes, comma separated")
     ap.add_argument("--arch-compare", default="",
                     help="livisun: instead of the RFQ workload, time prefill and decode of the "
                          "layer-list model beside the Llama decoder at equal layer sizes "

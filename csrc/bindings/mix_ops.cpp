@@ -29,7 +29,7 @@ bool launch_attn_mixq_prefill(bool, const float*, const void*, const void*, cons
                               const int32_t*, const int32_t*, const int32_t*, const int32_t*,
                               const int32_t*, int, void*, int64_t, const float*, const float*, int,
                               int, int, int, int, int, hipStream_t);
-bool launch_attn_mixq_prefill_mfma(const float*, const void*, const void*, const int32_t*, int,
+bool launch_attn_mixq_prefill_mfma(const float*, const float*, const void*, const void*, const int32_t*, int,
                                    const int32_t*, const int32_t*, const int32_t*, const int32_t*,
                                    const int32_t*, int, void*, int64_t, const float*, const float*,
                                    int, int, int, int, int, int, hipStream_t);
@@ -178,7 +178,7 @@ void attn_mixq_prefill(const Tensor& qmix, const Tensor& k_cache, const Tensor& 
                        const Tensor& bt, const Tensor& q_start, const Tensor& q_len,
                        const Tensor& kv_len, const Tensor& work_seq, const Tensor& work_qblk,
                        const Tensor& out, const Tensor& slopes, const OptT& sink, int64_t chunk,
-                       int64_t qblk, int64_t mfma) {
+                       int64_t qblk) {
   const bool f32 = act_f32(k_cache, "attn_mixq_prefill k_cache");
   TORCH_CHECK(qmix.dim() == 3, "attn_mixq_prefill: qmix [T, H, G dim]");
   const int H = (int)qmix.size(1), G = (int)k_cache.size(1), dim = (int)k_cache.size(3);
@@ -194,15 +194,6 @@ void attn_mixq_prefill(const Tensor& qmix, const Tensor& k_cache, const Tensor& 
               "attn_mixq_prefill: out [T, H vdim]");
   TORCH_CHECK(bt.dim() == 2 && bt.size(0) == NB, "attn_mixq_prefill: block_tables [NB, maxb]");
   const float* sk = optf(sink, "sink", H);
-  if (mfma && !f32) {
-    const bool ok = rfqmix::launch_attn_mixq_prefill_mfma(
-        f32p(qmix, "qmix"), k_cache.data_ptr(), v_cache.data_ptr(), i32p(bt, "block_tables", 0),
-        (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
-        i32p(kv_len, "kv_len", NB), i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W),
-        W, out.data_ptr(), out.stride(0), f32p(slopes, "slopes", H), sk, (int)chunk, H, G, dim,
-        vdim, BS, stream());
-    if (ok) return;
-  }
   const bool ok = rfqmix::launch_attn_mixq_prefill(
       f32, f32p(qmix, "qmix"), k_cache.data_ptr(), v_cache.data_ptr(), i32p(bt, "block_tables", 0),
       (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
@@ -210,6 +201,37 @@ void attn_mixq_prefill(const Tensor& qmix, const Tensor& k_cache, const Tensor& 
       out.data_ptr(), out.stride(0), f32p(slopes, "slopes", H), sk, (int)chunk, H, G, dim, vdim, BS,
       stream());
   TORCH_CHECK(ok, "attn_mixq_prefill: value size does not fit the LDS");
+}
+
+// The same attention on MFMA tiles (bf16 caches): takes the normed queries [T, H, dim] and the
+// scaled mixing matrix [H, H]; the mixed queries are formed in registers.
+void attn_mix_mfma(const Tensor& qn, const Tensor& ts, const Tensor& k_cache, const Tensor& v_cache,
+                   const Tensor& bt, const Tensor& q_start, const Tensor& q_len,
+                   const Tensor& kv_len, const Tensor& work_seq, const Tensor& work_qblk,
+                   const Tensor& out, const Tensor& slopes, const OptT& sink, int64_t chunk) {
+  TORCH_CHECK(!act_f32(k_cache, "attn_mix_mfma k_cache"), "attn_mix_mfma: bf16 caches");
+  TORCH_CHECK(qn.dim() == 3 && k_cache.dim() == 4 && v_cache.dim() == 4, "attn_mix_mfma: qn [T, H, dim]");
+  const int H = (int)qn.size(1), G = (int)k_cache.size(1), dim = (int)k_cache.size(3);
+  const int vdim = (int)v_cache.size(3), BS = (int)k_cache.size(2), NB = (int)q_len.numel();
+  const int W = (int)work_seq.numel();
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() && qn.size(2) == dim &&
+              v_cache.size(1) == G && v_cache.size(2) == BS &&
+              v_cache.scalar_type() == at::kBFloat16 && v_cache.size(0) == k_cache.size(0),
+              "attn_mix_mfma: caches [blocks, G, BS, dim | vdim]");
+  TORCH_CHECK(rfqmix::mixq_mfma_ok(H, G, dim, vdim, BS), "attn_mix_mfma: sizes outside the tiles");
+  TORCH_CHECK(out.scalar_type() == at::kBFloat16 && out.dim() == 2 && out.size(0) == qn.size(0) &&
+              out.size(1) == (int64_t)H * vdim && out.stride(1) == 1 && out.stride(0) % 4 == 0,
+              "attn_mix_mfma: out [T, H vdim]");
+  TORCH_CHECK(bt.dim() == 2 && bt.size(0) == NB, "attn_mix_mfma: block_tables [NB, maxb]");
+  TORCH_CHECK(work_qblk.numel() >= W, "attn_mix_mfma: work lists");
+  const bool ok = rfqmix::launch_attn_mixq_prefill_mfma(
+      f32p(qn, "qn"), f32p(ts, "talk_scaled", (int64_t)H * H), k_cache.data_ptr(),
+      v_cache.data_ptr(), i32p(bt, "block_tables", 0), (int)bt.size(1),
+      i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB), i32p(kv_len, "kv_len", NB),
+      i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W), W, out.data_ptr(),
+      out.stride(0), f32p(slopes, "slopes", H), optf(sink, "sink", H), (int)chunk, H, G, dim, vdim,
+      BS, stream());
+  TORCH_CHECK(ok, "attn_mix_mfma: no tile for these sizes");
 }
 
 bool mixq_mfma_ok(int64_t H, int64_t G, int64_t dim, int64_t vdim, int64_t BS) {
@@ -235,7 +257,8 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("canon_conv(Tensor h, Tensor w, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor(b!) out) -> ()");
   m.def("head_norm_append(Tensor qkv, Tensor q_w, Tensor k_w, float eps, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, int H, int G, int dim, int vdim, Tensor(c!) qn, Tensor? ts, Tensor(d!)? qmix, int mix_from) -> ()");
   m.def("attn_talk_decode(Tensor qn, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor(a!) out, Tensor slopes, Tensor? talk, Tensor? sink, float scale, int chunk, int max_rows) -> ()");
-  m.def("attn_mixq_prefill(Tensor qmix, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor slopes, Tensor? sink, int chunk, int qblk, int mfma) -> ()");
+  m.def("attn_mixq_prefill(Tensor qmix, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor slopes, Tensor? sink, int chunk, int qblk) -> ()");
+  m.def("attn_mix_mfma(Tensor qn, Tensor ts, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor slopes, Tensor? sink, int chunk) -> ()");
   m.def("glu_clamped(Tensor gate_up, float limit, float alpha, Tensor(a!) out) -> ()");
   m.def("mixq_mfma_ok", &mixq_mfma_ok);
 }
@@ -247,5 +270,6 @@ TORCH_LIBRARY_IMPL(rfq_mix, CUDA, m) {
   m.impl("head_norm_append", &head_norm_append);
   m.impl("attn_talk_decode", &attn_talk_decode);
   m.impl("attn_mixq_prefill", &attn_mixq_prefill);
+  m.impl("attn_mix_mfma", &attn_mix_mfma);
   m.impl("glu_clamped", &glu_clamped);
 }

@@ -1,19 +1,24 @@
-// MFMA form of attn_mixq_prefill for bf16 models (the math is at the top of mix_attn.hip).
+// MFMA attention of the layer-list models for bf16 caches (the math is at the top of
+// mix_attn.hip).
 //
-// Queries arrive mixed and scaled, [T, H, E] with E = G * dim, so the mixed score of head h
-// is ONE product with the concatenation of all G key heads, and every head of a token reads
-// the same keys.  A work item is (sequence, block of 32 query tokens, key/value head c); its
-// columns are the (token, head) pairs of the heads that use value head c, 16 per wave:
+// Head mixing is linear in the queries: with q~[h, c] = sum_{g in group c} (scale talk[h, g]) q_g
+// the mixed score of head h is ONE product of q~[h, :] (E = G * dim wide) with the
+// concatenation of all G key heads, and every head of a token reads the same keys.  A work
+// item is (sequence, block of 32 query tokens, key/value head c); its columns are the
+// (token, head) pairs of the heads that use value head c, 16 per wave:
 //
-//   S^T[key, col]  = K_cat[key, :] . Q~[col, :]         v_mfma_f32_16x16x32_bf16, A = keys
-//   bias, block mask, online softmax per column (fp32; the sink is the initial state)
-//   O^T[dv, col]  += V_c^T[dv, key] . P^T[key, col]      A = V^T by transposed LDS reads,
+//   prologue       q~ of the lane's column from the normed queries and the scaled mixing
+//                  matrix, straight into B-operand registers (no mixed-query tensor in memory)
+//   per 32-key page, shared by the workgroup's waves through LDS:
+//     S^T[key, col]  = K_cat[key, :] . Q~[col, :]       v_mfma_f32_16x16x32_bf16, A = keys
+//     bias, block mask, online softmax per column (fp32; the sink is the initial state)
+//     O^T[dv, col]  += V_c^T[dv, key] . P^T[key, col]    A = V^T by transposed LDS reads,
 //                                                        P split into bf16 hi + lo parts so
 //                                                        the weights keep fp32's precision
 //
-// One key tile is one 32-token page.  The waves of a workgroup share the page's V tile in
-// LDS; K fragments go straight from the cache to registers (16 B per lane).  The same kernel
-// serves the decode section (one token x rep heads per column tile).
+// K rows are padded by 64 B in LDS so that the 16 rows of an A fragment fall into different
+// banks.  Two workgroups fit a compute unit (LDS and registers): one loads while the other
+// multiplies.  The same kernel serves the decode section (one token x rep heads per tile).
 #include "common.h"
 
 namespace rfqmix {
@@ -21,18 +26,21 @@ namespace rfqmix {
 using namespace rfq;
 
 constexpr int kPg = 32;
+constexpr int kKPad = 32;          // bf16 elements of padding per K row in LDS
 
 template <int EK, int VT>
-__global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
-    const float* __restrict__ qmix, const bf16_t* __restrict__ k_cache,
+__global__ __launch_bounds__(256, 2) void attn_mixq_mfma_kernel(
+    const float* __restrict__ qn, const float* __restrict__ ts, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int maxb,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
     const int32_t* __restrict__ kv_len, const int32_t* __restrict__ work_seq,
     const int32_t* __restrict__ work_qblk, bf16_t* __restrict__ out, int64_t out_stride,
     const float* __restrict__ slopes, const float* __restrict__ sink, int chunk, int H, int G,
     int dim) {
-  constexpr int VD = VT * 16, E = EK * 32;
-  __shared__ __attribute__((aligned(16))) bf16_t v_lds[kPg * VD];
+  constexpr int VD = VT * 16, E = EK * 32, RS = E + kKPad;
+  extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
+  bf16_t* k_lds = lds;                       // [32][RS]
+  bf16_t* v_lds = lds + kPg * RS;            // [32][VD]
   const int s = work_seq[blockIdx.x];
   if (s < 0) return;
   const int ql = q_len[s], kl = kv_len[s];
@@ -41,6 +49,7 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
   const int nq = min(32, ql - i0);
   const int cg = blockIdx.y, rep = H / G;
   const int nwaves = blockDim.x >> 6, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (blockIdx.z * nwaves * 16 >= nq * rep) return;     // no column of this workgroup is used
   const int g4 = lane >> 4, c = lane & 15;
   const int tile = blockIdx.z * nwaves + wave;
   const bool active = tile * 16 < nq * rep;             // wave-uniform
@@ -52,40 +61,49 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
   const int ci = chunk > 0 ? pi / chunk : 0;
   const int jlo = chunk > 0 ? (p0 / chunk) * chunk : 0;
   const int32_t* bt = block_tables + (int64_t)s * maxb;
-  const float slope = slopes[hh < H ? hh : 0];
+  const float slope = slopes[hh];
 
   // mixed queries of this lane's column as B operands (k = 8 g4 + j of every 32-slice)
   s16x8 qf[EK];
   {
-    const float* qr = qmix + ((int64_t)(q_start[s] + i0 + (cvalid ? tok : 0)) * H + (cvalid ? hh : 0)) * E;
+    const float* qt = qn + (int64_t)(q_start[s] + i0 + (cvalid ? tok : 0)) * H * dim;
+    const float* tr = ts + (int64_t)hh * H;
 #pragma unroll
     for (int ks = 0; ks < EK; ++ks) {
-      float f[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) f[j] = cvalid ? qr[32 * ks + 8 * g4 + j] : 0.f;
+      const int e0 = 32 * ks + 8 * g4, ck = e0 / dim, x0 = e0 - ck * dim;
+      float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (cvalid)
+        for (int r = 0; r < rep; ++r) {
+          const float w = tr[ck * rep + r];
+          const float4* q4p = reinterpret_cast<const float4*>(qt + (int64_t)(ck * rep + r) * dim + x0);
+          const float4 a = q4p[0], b = q4p[1];
+          f[0] += w * a.x; f[1] += w * a.y; f[2] += w * a.z; f[3] += w * a.w;
+          f[4] += w * b.x; f[5] += w * b.y; f[6] += w * b.z; f[7] += w * b.w;
+        }
       qf[ks] = pack8(f);
     }
   }
-  // element offset of every 32-slice of the concatenated key inside a page (wave-uniform)
-  int koff[EK];
-#pragma unroll
-  for (int ks = 0; ks < EK; ++ks) {
-    const int ck = (32 * ks) / dim;
-    koff[ks] = ck * kPg * dim + (32 * ks - ck * dim);
-  }
-  const int klane = c * dim + 8 * g4;
   f32x4 o[VT];
 #pragma unroll
   for (int m = 0; m < VT; ++m) o[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
   float m_run = (sink != nullptr && cvalid) ? sink[hh] : -INFINITY;
   float l_run = (sink != nullptr && cvalid) ? 1.f : 0.f;
+  const bf16_t* ka = k_lds + c * RS + 8 * g4;          // this lane's A-fragment rows
 
   for (int pg = jlo / kPg; pg <= plast / kPg; ++pg) {
     const int kt = pg * kPg;
     const int64_t page = bt[pg];
-    // V tile of value head cg -> LDS; rows past the last written key are zeroed (they may
-    // hold anything, and 0 * NaN would poison the sum)
+    // K tile: the page's G key heads side by side, one LDS row per key
     {
+      const bf16_t* kb = k_cache + page * G * kPg * (int64_t)dim;
+      const int d8 = dim >> 3;
+      for (int x = threadIdx.x; x < kPg * (E / 8); x += blockDim.x) {
+        const int ck = x / (kPg * d8), rem = x - ck * kPg * d8, key = rem / d8, x8 = rem - key * d8;
+        const s16x8 v = reinterpret_cast<const s16x8*>(kb)[x];
+        *reinterpret_cast<s16x8*>(k_lds + key * RS + ck * dim + 8 * x8) = v;
+      }
+      // V tile of value head cg; rows past the last written key are zeroed (they may hold
+      // anything, and 0 * NaN would poison the sum)
       const bf16_t* vb = v_cache + ((page * G + cg) * kPg) * (int64_t)VD;
       for (int x = threadIdx.x; x < kPg * VD / 8; x += blockDim.x) {
         const int row = x / (VD / 8);
@@ -94,17 +112,15 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
         reinterpret_cast<s16x8*>(v_lds)[x] = v;
       }
     }
-    s16x8 pb_hi = (s16x8){0, 0, 0, 0, 0, 0, 0, 0}, pb_lo = pb_hi;
-    float alpha = 1.f;
+    __syncthreads();                                   // tiles visible
     if (active) {
       f32x4 sc[2];
-      const bf16_t* kp = k_cache + page * G * kPg * (int64_t)dim + klane;
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
         sc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < EK; ++ks) {
-          const s16x8 kf = *reinterpret_cast<const s16x8*>(kp + koff[ks] + 16 * mt * dim);
+          const s16x8 kf = *reinterpret_cast<const s16x8*>(ka + 16 * mt * RS + 32 * ks);
           sc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[ks]),
                                                            sc[mt], 0, 0, 0);
         }
@@ -125,7 +141,7 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m_run, mx);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      alpha = __expf(m_run - m_use);
+      const float alpha = __expf(m_run - m_use);
       float psum = 0.f, ph[8], pl[8];
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
@@ -139,11 +155,7 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
       l_run = l_run * alpha + psum;
       m_run = m_new;
       // P^T as B operand: element j <-> key (j < 4 ? 4 g4 + j : 16 + 4 g4 + j - 4)
-      pb_hi = pack8(ph);
-      pb_lo = pack8(pl);
-    }
-    __syncthreads();                                   // V tile visible
-    if (active) {
+      const s16x8 pb_hi = pack8(ph), pb_lo = pack8(pl);
       const int q4 = c >> 2, p4 = c & 3;
 #pragma unroll
       for (int m = 0; m < VT; ++m) {
@@ -156,7 +168,7 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
         o[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(pb_lo), o[m], 0, 0, 0);
       }
     }
-    __syncthreads();                                   // before the next page overwrites it
+    __syncthreads();                                   // before the next page overwrites the tiles
   }
   if (!cvalid) return;
   // lane holds O^T[dv = 16 m + 4 g4 + i][column c]
@@ -172,7 +184,7 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
 }
 
 template <int EK, int VT>
-static void launch_one(const float* qmix, const bf16_t* k, const bf16_t* v, const int32_t* bt,
+static void launch_one(const float* qn, const float* ts, const bf16_t* k, const bf16_t* v, const int32_t* bt,
                        int maxb, const int32_t* q_start, const int32_t* q_len,
                        const int32_t* kv_len, const int32_t* work_seq, const int32_t* work_qblk,
                        int W, bf16_t* out, int64_t out_stride, const float* slopes,
@@ -180,8 +192,15 @@ static void launch_one(const float* qmix, const bf16_t* k, const bf16_t* v, cons
   const int rep = H / G;
   const int nwaves = 2 * rep < 4 ? 2 * rep : 4;
   const int z = (2 * rep + nwaves - 1) / nwaves;
-  hipLaunchKernelGGL((attn_mixq_mfma_kernel<EK, VT>), dim3(W, G, z), dim3(nwaves * 64), 0, s, qmix,
-                     k, v, bt, maxb, q_start, q_len, kv_len, work_seq, work_qblk, out, out_stride,
+  const size_t lds = ((size_t)kPg * (EK * 32 + kKPad) + (size_t)kPg * VT * 16) * sizeof(bf16_t);
+  static bool attr = false;
+  if (!attr) {          // dynamic LDS above 64 KB has to be allowed per kernel, once
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mixq_mfma_kernel<EK, VT>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    attr = true;
+  }
+  hipLaunchKernelGGL((attn_mixq_mfma_kernel<EK, VT>), dim3(W, G, z), dim3(nwaves * 64), lds, s, qn,
+                     ts, k, v, bt, maxb, q_start, q_len, kv_len, work_seq, work_qblk, out, out_stride,
                      slopes, sink, chunk, H, G, dim);
 }
 
@@ -194,7 +213,7 @@ bool mixq_mfma_ok(int H, int G, int dim, int vdim, int BS) {
          (vdim == 32 || vdim == 64 || vdim == 128) && G <= 65535;
 }
 
-bool launch_attn_mixq_prefill_mfma(const float* qmix, const void* k_cache, const void* v_cache,
+bool launch_attn_mixq_prefill_mfma(const float* qn, const float* ts, const void* k_cache, const void* v_cache,
                                    const int32_t* bt, int maxb, const int32_t* q_start,
                                    const int32_t* q_len, const int32_t* kv_len,
                                    const int32_t* work_seq, const int32_t* work_qblk, int W,
@@ -206,7 +225,7 @@ bool launch_attn_mixq_prefill_mfma(const float* qmix, const void* k_cache, const
   const int EK = G * dim / 32, VT = vdim / 16;
 #define MIXQ_CASE(ek, vt)                                                                       \
   if (EK == ek && VT == vt) {                                                                   \
-    launch_one<ek, vt>(qmix, (const bf16_t*)k_cache, (const bf16_t*)v_cache, bt, maxb, q_start, \
+    launch_one<ek, vt>(qn, ts, (const bf16_t*)k_cache, (const bf16_t*)v_cache, bt, maxb, q_start, \
                        q_len, kv_len, work_seq, work_qblk, W, (bf16_t*)out, out_stride, slopes, \
                        sink, chunk, H, G, dim, s);                                              \
     return true;                                                                                \

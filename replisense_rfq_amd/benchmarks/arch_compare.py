@@ -74,7 +74,10 @@ def run(args) -> dict:
     g = torch.Generator().manual_seed(args.seed)
     out = {"layers": LAYERS, "vocab": VOCAB, "block": CHUNK, "prompt": [8, 2048],
            "decode": [64, 128], "sizes": {}}
+    only = [x for x in getattr(args, "arch_sizes", "").split(",") if x]
     for name, d, H, G, F in SIZES:
+        if only and name not in only:
+            continue
         row = {}
         for mcfg in _configs(name, d, H, G, F):
             kind = "livisun" if isinstance(mcfg, LayeredConfig) else "llama"

@@ -15,6 +15,7 @@ rows]`` (ForwardMeta) like the other decoders:
     attention: scale q.k - slope_h (i - j), mixed over heads, block mask, sink
        decode / short rows: attn_talk_decode (mixes raw scores in LDS)
        prefill rows:        attn_mixq_prefill (queries pre-mixed, keys concatenated)
+       bf16 with head sizes of the MFMA tiles: attn_mix_mfma for both sections
     o GEMM ; x += rms(y) w1b ls1 ; h = rms(x) w2          (one kernel)
     conv ; gate|up GEMM ; clamped GLU ; down GEMM ; x += rms(y) w2b ls2
   final norm on the rows that need logits -> head GEMM (fp32 logits).
@@ -126,25 +127,30 @@ class LivisunLM:
             ops.canon_conv(h, lw["canon1"], self.state[li, 0], rs, rb, rf, pos, hc)
             qkv = ops.matmul_nt(hc, lw["qkv"])
             qn = torch.empty((T, H, dim), dtype=torch.float32, device=dev)
-            mix_from = 0 if lw["mixq_decode"] else D
+            mfma = lw["mixq_decode"]           # queries stay unmixed: the kernel mixes them
+            mix_from = T if mfma else D
             qmix = torch.empty((T - mix_from, H, G * dim), dtype=torch.float32, device=dev) \
                 if T > mix_from else None
             ops.head_norm_append(qkv, lw["q_norm"], lw["k_norm"], eps, m.slot_mapping[:T],
                                  self.kv_k[li], self.kv_v[li], H, G, dim, vd, qn,
                                  lw["talk_scaled"], qmix, mix_from)
             attn = torch.empty((T, H * vd), dtype=dt, device=dev)
-            if D > 0 and lw["mixq_decode"]:
-                NA = m.dec_q_len.shape[0]
-                ids, zeros = self._decode_work(NA)
-                ops.attn_mixq_prefill(qmix[:D], self.kv_k[li], self.kv_v[li], m.dec_block_tables,
-                                      m.dec_q_start, m.dec_q_len, m.dec_kv_len, ids, zeros,
-                                      attn[:D], lw["slopes_mixed"], lw["sink"], mx.chunk)
+            if D > 0 and mfma:
+                ids, zeros = self._decode_work(m.dec_q_len.shape[0])
+                ops.attn_mix_mfma(qn[:D], lw["talk_scaled"], self.kv_k[li], self.kv_v[li],
+                                  m.dec_block_tables, m.dec_q_start, m.dec_q_len, m.dec_kv_len,
+                                  ids, zeros, attn[:D], lw["slopes_mixed"], lw["sink"], mx.chunk)
             elif D > 0:
                 ops.attn_talk_decode(qn[:D], self.kv_k[li], self.kv_v[li], m.dec_block_tables,
                                      m.dec_q_start, m.dec_q_len, m.dec_kv_len, attn[:D],
                                      lw["slopes"], lw["talk"], lw["sink"], mx.scale, mx.chunk)
-            if T > D:
-                ops.attn_mixq_prefill(qmix[D - mix_from:], self.kv_k[li], self.kv_v[li], m.pf_block_tables,
+            if T > D and mfma:
+                ops.attn_mix_mfma(qn[D:], lw["talk_scaled"], self.kv_k[li], self.kv_v[li],
+                                  m.pf_block_tables, m.pf_q_start, m.pf_q_len, m.pf_kv_len,
+                                  m.work_seq, m.work_qblk, attn[D:T], lw["slopes_mixed"],
+                                  lw["sink"], mx.chunk)
+            elif T > D:
+                ops.attn_mixq_prefill(qmix, self.kv_k[li], self.kv_v[li], m.pf_block_tables,
                                       m.pf_q_start, m.pf_q_len, m.pf_kv_len, m.work_seq,
                                       m.work_qblk, attn[D:T], lw["slopes_mixed"], lw["sink"],
                                       mx.chunk, m.prefill_qblk)

@@ -1096,9 +1096,26 @@ def attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len, kv_l
     if _gpu(qmix):
         _native.mix_ops().attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len,
                                             kv_len, work_seq, work_qblk, out, slopes, sink,
-                                            int(chunk), int(qblk), int(MIXQ_MFMA))
+                                            int(chunk), int(qblk))
     else:
         ref.attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len, kv_len, out,
+                              slopes, sink, chunk)
+
+
+def attn_mix_mfma(qn, talk_scaled, k_cache, v_cache, block_tables, q_start, q_len, kv_len,
+                  work_seq, work_qblk, out, slopes, sink, chunk: int):
+    """attn_mixq_prefill on MFMA tiles (bf16 caches, sizes of mixq_mfma_ok): the queries come
+    normed but unmixed, [T, H, dim]; the kernel mixes them in registers."""
+    if _gpu(qn):
+        _native.mix_ops().attn_mix_mfma(qn, talk_scaled, k_cache, v_cache, block_tables, q_start,
+                                        q_len, kv_len, work_seq, work_qblk, out, slopes, sink,
+                                        int(chunk))
+    else:
+        T, H, dim = qn.shape
+        G = k_cache.shape[1]
+        qm = torch.einsum("hcr,tcrd->thcd", talk_scaled.float().view(H, G, H // G),
+                          qn.view(T, G, H // G, dim)).reshape(T, H, G * dim)
+        ref.attn_mixq_prefill(qm, k_cache, v_cache, block_tables, q_start, q_len, kv_len, out,
                               slopes, sink, chunk)
 
 

@@ -138,14 +138,18 @@ def test_attn_talk_decode(dt, H, G, dim, vdim, chunk, use_talk, use_sink):
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,dim,vdim,chunk", CASES + [(2, 2, 64, 64, 0), (8, 2, 128, 128, 96)])
 @pytest.mark.parametrize("mfma", [False, True])
-def test_attn_mixq_prefill(dt, H, G, dim, vdim, chunk, mfma, monkeypatch):
+def test_attn_mixq_prefill(dt, H, G, dim, vdim, chunk, mfma):
     if mfma and dt != torch.bfloat16:
         pytest.skip("the MFMA tiles are bf16")
-    monkeypatch.setattr(ops, "MIXQ_MFMA", mfma)
+    if mfma and not ops.mixq_mfma_ok(H, G, dim, vdim):
+        pytest.skip("sizes outside the MFMA tiles")
     lens, qlens = [33, 300, 97, 64, 2], [33, 120, 40, 64, 2]
     g, kc, vc, m = _paged(dt, H, G, dim, vdim, lens, qlens, 6)
     T = sum(qlens)
-    qmix = torch.randn(T, H, G * dim, generator=g) * 0.2
+    qn = torch.randn(T, H, dim, generator=g)
+    ts = (torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)) * 0.2
+    qmix = torch.einsum("hcr,tcrd->thcd", ts.view(H, G, H // G),
+                        qn.view(T, G, H // G, dim)).reshape(T, H, G * dim).contiguous()
     slopes = torch.rand(H, generator=g) * 0.2
     sink = torch.randn(H, generator=g)
     ws, wq = [], []
@@ -158,9 +162,12 @@ def test_attn_mixq_prefill(dt, H, G, dim, vdim, chunk, mfma, monkeypatch):
     ref.attn_mixq_prefill(qmix, kc, vc, m["bt"], m["q_start"], m["q_len"], m["kv_len"], want,
                           slopes, sink, chunk)
     got = torch.empty(T, H * vdim, dtype=dt, device=DEV)
-    ops.attn_mixq_prefill(qmix.to(DEV), kc.to(DEV), vc.to(DEV), m["bt"].to(DEV),
-                          m["q_start"].to(DEV), m["q_len"].to(DEV), m["kv_len"].to(DEV),
-                          ws.to(DEV), wq.to(DEV), got, slopes.to(DEV), sink.to(DEV), chunk)
+    args = (kc.to(DEV), vc.to(DEV), m["bt"].to(DEV), m["q_start"].to(DEV), m["q_len"].to(DEV),
+            m["kv_len"].to(DEV), ws.to(DEV), wq.to(DEV), got, slopes.to(DEV), sink.to(DEV), chunk)
+    if mfma:
+        ops.attn_mix_mfma(qn.to(DEV), ts.to(DEV), *args)
+    else:
+        ops.attn_mixq_prefill(qmix.to(DEV), *args)
     torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
 
 
