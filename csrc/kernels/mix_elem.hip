@@ -21,10 +21,79 @@ __global__ __launch_bounds__(256) void embed_sinusoid_kernel(
   const T* row = table + (int64_t)id * d;
   const float p = (float)pos[t];
   float* o = out + (int64_t)t * d;
-  for (int c = threadIdx.x; c < d; c += blockDim.x) {
-    const float ang = p * inv_freq[c >> 1];
-    const float pe = (c & 1) ? cosf(ang) : sinf(ang);
-    o[c] = ldf(row + c) * scale + pe;
+  for (int i = threadIdx.x; 2 * i < d; i += blockDim.x) {
+    float sn, cs;
+    sincosf(p * inv_freq[i], &sn, &cs);
+    o[2 * i] = ldf(row + 2 * i) * scale + sn;
+    if (2 * i + 1 < d) o[2 * i + 1] = ldf(row + 2 * i + 1) * scale + cs;
+  }
+}
+
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 ld4(const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
+                     __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+}
+__device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void st4(bf16_t* p, float4 v) {
+  bf16_t t[4];
+  stf(t, v.x); stf(t + 1, v.y); stf(t + 2, v.z); stf(t + 3, v.w);
+  *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(t);
+}
+
+// The same with the row held in registers: d a multiple of 4, at most NCH * 1024.  Every
+// operand is read once, in 16-byte pieces, before the first reduction.
+template <typename T, int NCH>
+__global__ __launch_bounds__(256) void sandwich_norm_vec_kernel(
+    const T* __restrict__ y, int64_t y_stride, float* __restrict__ residual,
+    const float* __restrict__ w_post, const float* __restrict__ gain,
+    const float* __restrict__ w_pre, float* __restrict__ out, int d, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  float* x = residual + (int64_t)t * d;
+  float4 xv[NCH], yv[NCH], wn[NCH];
+  float sy = 0.f;
+#pragma unroll
+  for (int k = 0; k < NCH; ++k) {
+    const int c = (threadIdx.x + k * 256) * 4;
+    if (c < d) {
+      xv[k] = ld4(x + c);
+      wn[k] = ld4(w_pre + c);
+      if (y != nullptr) {
+        const float4 a = ld4(y + (int64_t)t * y_stride + c), p = ld4(w_post + c), g = ld4(gain + c);
+        sy += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+        yv[k] = make_float4(a.x * p.x * g.x, a.y * p.y * g.y, a.z * p.z * g.z, a.w * p.w * g.w);
+      }
+    }
+  }
+  float ss = 0.f;
+  if (y != nullptr) {
+    sy = block_sum(sy, scratch);
+    const float ry = 1.0f / sqrtf(sy / (float)d + eps);
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+      const int c = (threadIdx.x + k * 256) * 4;
+      if (c < d) {
+        xv[k].x += yv[k].x * ry; xv[k].y += yv[k].y * ry;
+        xv[k].z += yv[k].z * ry; xv[k].w += yv[k].w * ry;
+        st4(x + c, xv[k]);
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NCH; ++k)
+    if ((threadIdx.x + k * 256) * 4 < d)
+      ss += xv[k].x * xv[k].x + xv[k].y * xv[k].y + xv[k].z * xv[k].z + xv[k].w * xv[k].w;
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)d + eps);
+  float* o = out + (int64_t)t * d;
+#pragma unroll
+  for (int k = 0; k < NCH; ++k) {
+    const int c = (threadIdx.x + k * 256) * 4;
+    if (c < d)
+      st4(o + c, make_float4(xv[k].x * r * wn[k].x, xv[k].y * r * wn[k].y, xv[k].z * r * wn[k].z,
+                             xv[k].w * r * wn[k].w));
   }
 }
 
@@ -102,12 +171,49 @@ __global__ __launch_bounds__(256) void canon_conv_kernel(
   }
 }
 
+// Four channels per thread (d a multiple of 4): 16-byte loads of h and of the state.
+template <typename T>
+__global__ __launch_bounds__(256) void canon_conv_vec_kernel(
+    const float* __restrict__ h, const float* __restrict__ w, float* __restrict__ state,
+    const int32_t* __restrict__ row_state, const int32_t* __restrict__ row_back,
+    const int32_t* __restrict__ row_fwd, const int32_t* __restrict__ pos, T* __restrict__ out,
+    int d, int taps, int slots) {
+  const int t = blockIdx.x;
+  const int code = row_state[t], i = row_back[t], f = row_fwd[t], p = pos[t];
+  const int K = taps - 1;
+  const float* rd = code >= 0 ? state + ((int64_t)((code & 1) * slots + (code >> 1)) * K) * d : nullptr;
+  float* wr = code >= 0 ? state + ((int64_t)((1 - (code & 1)) * slots + (code >> 1)) * K) * d : nullptr;
+  const float* hr = h + (int64_t)t * d;
+  const int q = i + f + 1;
+  for (int c = threadIdx.x * 4; c < d; c += blockDim.x * 4) {
+    const float4 h0 = ld4(hr + c);
+    const float* wc = w + (int64_t)c * taps;             // [4][taps]
+    float4 acc = make_float4(h0.x + wc[taps - 1] * h0.x, h0.y + wc[2 * taps - 1] * h0.y,
+                             h0.z + wc[3 * taps - 1] * h0.z, h0.w + wc[4 * taps - 1] * h0.w);
+    for (int dl = 1; dl < taps; ++dl) {
+      float4 src;
+      if (dl <= i) src = ld4(hr + c - (int64_t)dl * d);
+      else if (p - dl >= 0 && rd != nullptr) src = ld4(rd + (int64_t)(K + i - dl) * d + c);
+      else continue;
+      const int j = taps - 1 - dl;
+      acc.x += wc[j] * src.x; acc.y += wc[taps + j] * src.y;
+      acc.z += wc[2 * taps + j] * src.z; acc.w += wc[3 * taps + j] * src.w;
+    }
+    st4(out + (int64_t)t * d + c, acc);
+    if (wr != nullptr) {
+      if (f < K) st4(wr + (int64_t)(K - 1 - f) * d + c, h0);
+      if (i == 0)
+        for (int e = 0; e < K - q; ++e) st4(wr + (int64_t)e * d + c, ld4(rd + (int64_t)(e + q) * d + c));
+    }
+  }
+}
+
 // One workgroup per token.  Wave w takes the head items w, w + nw, ...: q heads (rms norm
 // with weight -> qn fp32 and LDS), k heads (rms norm with weight -> paged cache), v heads
 // (unit rms -> paged cache).  Rows >= mix_from then write the mixed queries
 // qmix[t - mix_from][h][c * dim + x] = sum_r ts[h][c * rep + r] * qn[c * rep + r][x].
 template <typename T>
-__global__ __launch_bounds__(256) void head_norm_append_kernel(
+__global__ __launch_bounds__(1024) void head_norm_append_kernel(
     const T* __restrict__ qkv, int64_t stride, const float* __restrict__ q_w,
     const float* __restrict__ k_w, float eps, const int32_t* __restrict__ slots,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int dim, int vdim, int BS,
@@ -170,6 +276,28 @@ __global__ __launch_bounds__(256) void glu_clamped_kernel(const T* __restrict__ 
   stf(out + (int64_t)t * ostride + c, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
 }
 
+// Four columns per thread (F and the row strides multiples of 4).
+template <typename T>
+__global__ __launch_bounds__(256) void glu_clamped_vec_kernel(const T* __restrict__ gu,
+                                                              int64_t stride, T* __restrict__ out,
+                                                              int64_t ostride, int F, float limit,
+                                                              float alpha) {
+  const int t = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
+  if (c >= F) return;
+  const T* r = gu + (int64_t)t * stride;
+  const float4 g4 = ld4(r + c), u4 = ld4(r + F + c);
+  const float gs[4] = {g4.x, g4.y, g4.z, g4.w}, us[4] = {u4.x, u4.y, u4.z, u4.w};
+  float o[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float g = fminf(gs[k], limit);
+    const float u = fminf(fmaxf(us[k], -limit), limit);
+    o[k] = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+  }
+  st4(out + (int64_t)t * ostride + c, make_float4(o[0], o[1], o[2], o[3]));
+}
+
 // ------------------------------------------------------------------ launchers
 #define MIX_DISPATCH(f32, ...)              \
   do {                                      \
@@ -189,6 +317,18 @@ void launch_sandwich_norm(bool f32, const void* y, int64_t y_stride, float* resi
                           const float* w_post, const float* gain, const float* w_pre, float* out,
                           int T_, int d, float eps, hipStream_t s) {
   if (T_ == 0) return;
+  if (d % 4 == 0 && d <= 8192 && y_stride % 4 == 0) {
+#define SANDWICH_VEC(n)                                                                          \
+  MIX_DISPATCH(f32, hipLaunchKernelGGL((sandwich_norm_vec_kernel<T, n>), dim3(T_), dim3(256), 0, s, \
+                                       (const T*)y, y_stride, residual, w_post, gain, w_pre, out, d, \
+                                       eps))
+    if (d <= 1024) SANDWICH_VEC(1);
+    else if (d <= 2048) SANDWICH_VEC(2);
+    else if (d <= 4096) SANDWICH_VEC(4);
+    else SANDWICH_VEC(8);
+#undef SANDWICH_VEC
+    return;
+  }
   MIX_DISPATCH(f32, hipLaunchKernelGGL(sandwich_norm_kernel<T>, dim3(T_), dim3(256), 0, s,
                                        (const T*)y, y_stride, residual, w_post, gain, w_pre, out, d,
                                        eps));
@@ -199,6 +339,12 @@ void launch_canon_conv(bool f32, const float* h, const float* w, float* state,
                        const int32_t* pos, void* out, int T_, int d, int taps, int slots,
                        hipStream_t s) {
   if (T_ == 0) return;
+  if (d % 4 == 0) {
+    MIX_DISPATCH(f32, hipLaunchKernelGGL(canon_conv_vec_kernel<T>, dim3(T_), dim3(256), 0, s, h, w,
+                                         state, row_state, row_back, row_fwd, pos, (T*)out, d, taps,
+                                         slots));
+    return;
+  }
   MIX_DISPATCH(f32, hipLaunchKernelGGL(canon_conv_kernel<T>, dim3(T_), dim3(256), 0, s, h, w, state,
                                        row_state, row_back, row_fwd, pos, (T*)out, d, taps, slots));
 }
@@ -209,7 +355,8 @@ void launch_head_norm_append(bool f32, const void* qkv, int64_t stride, const fl
                              float* qn, const float* ts, float* qmix, int mix_from, hipStream_t s) {
   if (T_ == 0) return;
   const size_t lds = (size_t)H * dim * sizeof(float);       // checked <= 64 KB by the caller
-  MIX_DISPATCH(f32, hipLaunchKernelGGL(head_norm_append_kernel<T>, dim3(T_), dim3(256), lds, s,
+  const int threads = H + 2 * G >= 16 ? 1024 : 256;     // a wave per head item, up to 16 at once
+  MIX_DISPATCH(f32, hipLaunchKernelGGL(head_norm_append_kernel<T>, dim3(T_), dim3(threads), lds, s,
                                        (const T*)qkv, stride, q_w, k_w, eps, slots, (T*)k_cache,
                                        (T*)v_cache, H, G, dim, vdim, BS, qn, ts, qmix, mix_from));
 }
@@ -217,6 +364,12 @@ void launch_head_norm_append(bool f32, const void* qkv, int64_t stride, const fl
 void launch_glu_clamped(bool f32, const void* gu, int64_t stride, void* out, int64_t ostride,
                         int T_, int F, float limit, float alpha, hipStream_t s) {
   if (T_ == 0) return;
+  if (F % 4 == 0 && stride % 4 == 0 && ostride % 4 == 0) {
+    MIX_DISPATCH(f32, hipLaunchKernelGGL(glu_clamped_vec_kernel<T>, dim3(T_, (F / 4 + 255) / 256),
+                                         dim3(256), 0, s, (const T*)gu, stride, (T*)out, ostride, F,
+                                         limit, alpha));
+    return;
+  }
   MIX_DISPATCH(f32, hipLaunchKernelGGL(glu_clamped_kernel<T>, dim3(T_, (F + 255) / 256), dim3(256),
                                        0, s, (const T*)gu, stride, (T*)out, ostride, F, limit,
                                        alpha));
