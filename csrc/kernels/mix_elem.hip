@@ -42,6 +42,30 @@ __device__ __forceinline__ void st4(bf16_t* p, float4 v) {
   *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(t);
 }
 
+__device__ __forceinline__ void ld8(const float* p, float* f) {
+  const float4 a = ld4(p), b = ld4(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+__device__ __forceinline__ void ld8(const bf16_t* p, float* f) {
+  const uint4 v = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    f[2 * k] = __uint_as_float(w[k] << 16);
+    f[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ void st8(float* p, const float* f) {
+  st4(p, make_float4(f[0], f[1], f[2], f[3]));
+  st4(p + 4, make_float4(f[4], f[5], f[6], f[7]));
+}
+__device__ __forceinline__ void st8(bf16_t* p, const float* f) {
+  bf16_t t[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) stf(t + k, f[k]);
+  *reinterpret_cast<uint4*>(p) = *reinterpret_cast<const uint4*>(t);
+}
+
 // The same with the row held in registers: d a multiple of 4, at most NCH * 1024.  Every
 // operand is read once, in 16-byte pieces, before the first reduction.
 template <typename T, int NCH>
@@ -171,13 +195,17 @@ __global__ __launch_bounds__(256) void canon_conv_kernel(
   }
 }
 
-// Four channels per thread (d a multiple of 4): 16-byte loads of h and of the state.
-template <typename T>
+constexpr int kVecTaps = 4;      // most taps of the vector form (compiled per tap count)
+
+// Four channels per thread (d a multiple of 4, at most kVecTaps taps): 16-byte loads of h,
+// of the state and of the taps.
+template <typename T, int TAPS>
 __global__ __launch_bounds__(256) void canon_conv_vec_kernel(
     const float* __restrict__ h, const float* __restrict__ w, float* __restrict__ state,
     const int32_t* __restrict__ row_state, const int32_t* __restrict__ row_back,
     const int32_t* __restrict__ row_fwd, const int32_t* __restrict__ pos, T* __restrict__ out,
-    int d, int taps, int slots) {
+    int d, int slots) {
+  constexpr int taps = TAPS;
   const int t = blockIdx.x;
   const int code = row_state[t], i = row_back[t], f = row_fwd[t], p = pos[t];
   const int K = taps - 1;
@@ -187,9 +215,15 @@ __global__ __launch_bounds__(256) void canon_conv_vec_kernel(
   const int q = i + f + 1;
   for (int c = threadIdx.x * 4; c < d; c += blockDim.x * 4) {
     const float4 h0 = ld4(hr + c);
-    const float* wc = w + (int64_t)c * taps;             // [4][taps]
+    // the four channels' taps are 4 * taps contiguous floats: read them in 16-byte pieces
+    float wv[4 * TAPS];
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k)
+      *reinterpret_cast<float4*>(wv + 4 * k) = ld4(w + (int64_t)c * taps + 4 * k);
+    const float* wc = wv;                                // [4][taps]
     float4 acc = make_float4(h0.x + wc[taps - 1] * h0.x, h0.y + wc[2 * taps - 1] * h0.y,
                              h0.z + wc[3 * taps - 1] * h0.z, h0.w + wc[4 * taps - 1] * h0.w);
+#pragma unroll
     for (int dl = 1; dl < taps; ++dl) {
       float4 src;
       if (dl <= i) src = ld4(hr + c - (int64_t)dl * d);
@@ -223,6 +257,56 @@ __global__ __launch_bounds__(1024) void head_norm_append_kernel(
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const T* row = qkv + (int64_t)t * stride;
   const int slot = slots[t];
+  const int Lq = dim >> 3, Lv = vdim >> 3;
+  const bool vec = dim % 8 == 0 && vdim % 8 == 0 && Lq <= 64 && Lv <= 64 && (Lq & (Lq - 1)) == 0 &&
+                   (Lv & (Lv - 1)) == 0 && stride % 8 == 0;
+  if (vec) {
+    // 16-byte accesses: a head is dim / 8 (vdim / 8) lanes wide, several heads per wave pass
+    {
+      const int hp = 64 / Lq, sub = lane / Lq, li = lane - sub * Lq;
+      for (int base = wid * hp; base < H + G; base += nw * hp) {
+        const int it = base + sub;
+        const bool valid = it < H + G;
+        float f[8];
+        ld8(row + (int64_t)(valid ? it : 0) * dim + li * 8, f);
+        float ss = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) ss += f[k] * f[k];
+        for (int o = Lq >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        const float r = 1.0f / sqrtf(ss / (float)dim + eps);
+        float wv[8];
+        ld8((valid && it >= H) ? k_w + li * 8 : q_w + li * 8, wv);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) f[k] = f[k] * r * wv[k];
+        if (valid && it < H) {
+          st8(qn + ((int64_t)t * H + it) * dim + li * 8, f);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) qs[it * dim + li * 8 + k] = f[k];
+        } else if (valid && slot >= 0) {
+          st8(k_cache + (((int64_t)(slot / BS) * G + (it - H)) * BS + slot % BS) * (int64_t)dim + li * 8, f);
+        }
+      }
+    }
+    {
+      const int hp = 64 / Lv, sub = lane / Lv, li = lane - sub * Lv;
+      const T* vrow = row + (int64_t)(H + G) * dim;
+      for (int base = wid * hp; base < G; base += nw * hp) {
+        const int it = base + sub;
+        const bool valid = it < G;
+        float f[8];
+        ld8(vrow + (int64_t)(valid ? it : 0) * vdim + li * 8, f);
+        float ss = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) ss += f[k] * f[k];
+        for (int o = Lv >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        const float r = 1.0f / sqrtf(ss / (float)vdim + eps);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) f[k] *= r;
+        if (valid && slot >= 0)
+          st8(v_cache + (((int64_t)(slot / BS) * G + it) * BS + slot % BS) * (int64_t)vdim + li * 8, f);
+      }
+    }
+  } else
   for (int it = wid; it < H + 2 * G; it += nw) {
     const bool is_q = it < H, is_k = !is_q && it < H + G;
     const int n = (is_q || is_k) ? dim : vdim;
@@ -339,10 +423,16 @@ void launch_canon_conv(bool f32, const float* h, const float* w, float* state,
                        const int32_t* pos, void* out, int T_, int d, int taps, int slots,
                        hipStream_t s) {
   if (T_ == 0) return;
-  if (d % 4 == 0) {
-    MIX_DISPATCH(f32, hipLaunchKernelGGL(canon_conv_vec_kernel<T>, dim3(T_), dim3(256), 0, s, h, w,
-                                         state, row_state, row_back, row_fwd, pos, (T*)out, d, taps,
-                                         slots));
+  if (d % 4 == 0 && taps <= kVecTaps) {
+#define CANON_VEC(n)                                                                              \
+  MIX_DISPATCH(f32, hipLaunchKernelGGL((canon_conv_vec_kernel<T, n>), dim3(T_), dim3(256), 0, s, h, \
+                                       w, state, row_state, row_back, row_fwd, pos, (T*)out, d,   \
+                                       slots))
+    if (taps == 1) CANON_VEC(1);
+    else if (taps == 2) CANON_VEC(2);
+    else if (taps == 3) CANON_VEC(3);
+    else CANON_VEC(4);
+#undef CANON_VEC
     return;
   }
   MIX_DISPATCH(f32, hipLaunchKernelGGL(canon_conv_kernel<T>, dim3(T_), dim3(256), 0, s, h, w, state,

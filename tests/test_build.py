@@ -14,3 +14,14 @@ def test_native_libraries_build_and_load():
         assert hasattr(torch.ops.rfq_amd, op), op
     rt = runtime.load()
     assert hasattr(rt, "EngineCore") and hasattr(rt, "Grammar")
+
+
+def test_layer_list_kernel_library_builds_and_loads():
+    so = _build.build_mix_kernels()
+    torch.ops.load_library(str(so))
+    for op in ("embed_sinusoid", "sandwich_norm", "canon_conv", "head_norm_append",
+               "attn_talk_decode", "attn_mixq_prefill", "attn_mix_mfma", "glu_clamped",
+               "mixq_mfma_ok"):
+        assert hasattr(torch.ops.rfq_mix, op), op
+    assert torch.ops.rfq_mix.mixq_mfma_ok(32, 8, 128, 128, 32)
+    assert not torch.ops.rfq_mix.mixq_mfma_ok(6, 3, 24, 40, 32)
