@@ -16,8 +16,8 @@
 //                                                        P split into bf16 hi + lo parts so
 //                                                        the weights keep fp32's precision
 //
-// K rows are padded by 64 B in LDS so that the 16 rows of an A fragment fall into different
-// banks.  Two workgroups fit a compute unit (LDS and registers): one loads while the other
+// K and V rows are padded by 16 B in LDS so that the rows of a fragment read fall into
+// different banks.  Two workgroups fit a compute unit (LDS and registers): one loads while the other
 // multiplies.  The same kernel serves the decode section (one token x rep heads per tile).
 #include "common.h"
 
@@ -26,10 +26,12 @@ namespace rfqmix {
 using namespace rfq;
 
 constexpr int kPg = 32;
-constexpr int kKPad = 32;          // bf16 elements of padding per K row in LDS
+constexpr int kKPad = 8;           // bf16 elements of padding per K / V row in LDS: row strides
+                                   // of 16 B modulo 128 B, so the 8 lanes of a 16-byte read
+                                   // phase (rows c .. c + 7) fall into different banks
 
 template <int EK, int VT>
-__global__ __launch_bounds__(256, 2) void attn_mixq_mfma_kernel(
+__global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
     const float* __restrict__ qn, const float* __restrict__ ts, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int maxb,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
@@ -37,10 +39,10 @@ __global__ __launch_bounds__(256, 2) void attn_mixq_mfma_kernel(
     const int32_t* __restrict__ work_qblk, bf16_t* __restrict__ out, int64_t out_stride,
     const float* __restrict__ slopes, const float* __restrict__ sink, int chunk, int H, int G,
     int dim) {
-  constexpr int VD = VT * 16, E = EK * 32, RS = E + kKPad;
+  constexpr int VD = VT * 16, E = EK * 32, RS = E + kKPad, VRS = VD + kKPad;
   extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
   bf16_t* k_lds = lds;                       // [32][RS]
-  bf16_t* v_lds = lds + kPg * RS;            // [32][VD]
+  bf16_t* v_lds = lds + kPg * RS;            // [32][VRS]
   const int s = work_seq[blockIdx.x];
   if (s < 0) return;
   const int ql = q_len[s], kl = kv_len[s];
@@ -90,29 +92,54 @@ __global__ __launch_bounds__(256, 2) void attn_mixq_mfma_kernel(
   float l_run = (sink != nullptr && cvalid) ? 1.f : 0.f;
   const bf16_t* ka = k_lds + c * RS + 8 * g4;          // this lane's A-fragment rows
 
-  for (int pg = jlo / kPg; pg <= plast / kPg; ++pg) {
-    const int kt = pg * kPg;
-    const int64_t page = bt[pg];
-    // K tile: the page's G key heads side by side, one LDS row per key
-    {
-      const bf16_t* kb = k_cache + page * G * kPg * (int64_t)dim;
-      const int d8 = dim >> 3;
-      for (int x = threadIdx.x; x < kPg * (E / 8); x += blockDim.x) {
-        const int ck = x / (kPg * d8), rem = x - ck * kPg * d8, key = rem / d8, x8 = rem - key * d8;
-        const s16x8 v = reinterpret_cast<const s16x8*>(kb)[x];
-        *reinterpret_cast<s16x8*>(k_lds + key * RS + ck * dim + 8 * x8) = v;
-      }
-      // V tile of value head cg; rows past the last written key are zeroed (they may hold
-      // anything, and 0 * NaN would poison the sum)
-      const bf16_t* vb = v_cache + ((page * G + cg) * kPg) * (int64_t)VD;
-      for (int x = threadIdx.x; x < kPg * VD / 8; x += blockDim.x) {
-        const int row = x / (VD / 8);
-        s16x8 v = reinterpret_cast<const s16x8*>(vb)[x];
-        if (kt + row > plast) v = (s16x8){0, 0, 0, 0, 0, 0, 0, 0};
-        reinterpret_cast<s16x8*>(v_lds)[x] = v;
-      }
+  // Page pipeline: the next page's K / V pieces are loaded into registers while this page is
+  // multiplied out of LDS (one memory round trip per page, hidden behind the MFMAs).
+  constexpr int NK = (kPg * (E / 8) + 255) / 256, NV = (kPg * (VD / 8) + 255) / 256;
+  s16x8 kreg[NK], vreg[NV];
+  int kdst[NK];                                        // LDS element offset of every K piece
+  {
+    const int d8 = dim >> 3;
+#pragma unroll
+    for (int u = 0; u < NK; ++u) {
+      const int x = threadIdx.x + u * 256;
+      const int rowi = x / d8, x8 = x - rowi * d8, ck = rowi >> 5, key = rowi & 31;
+      kdst[u] = x < kPg * (E / 8) ? key * RS + ck * dim + 8 * x8 : -1;
     }
+  }
+  auto fetch = [&](int pg) {
+    const int64_t page = bt[pg];
+    const s16x8* kb = reinterpret_cast<const s16x8*>(k_cache + page * G * kPg * (int64_t)dim);
+    const s16x8* vb = reinterpret_cast<const s16x8*>(v_cache + ((page * G + cg) * kPg) * (int64_t)VD);
+#pragma unroll
+    for (int u = 0; u < NK; ++u)
+      if (kdst[u] >= 0) kreg[u] = kb[threadIdx.x + u * 256];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int x = threadIdx.x + u * 256;
+      // rows past the last written key are zeroed (they may hold anything, and 0 * NaN
+      // would poison the sum)
+      if (x < kPg * (VD / 8))
+        vreg[u] = pg * kPg + x / (VD / 8) > plast ? (s16x8){0, 0, 0, 0, 0, 0, 0, 0} : vb[x];
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int u = 0; u < NK; ++u)
+      if (kdst[u] >= 0) *reinterpret_cast<s16x8*>(k_lds + kdst[u]) = kreg[u];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int x = threadIdx.x + u * 256;
+      if (x < kPg * (VD / 8))
+        *reinterpret_cast<s16x8*>(v_lds + (x / (VD / 8)) * VRS + 8 * (x % (VD / 8))) = vreg[u];
+    }
+  };
+  const int pg_last = plast / kPg;
+  fetch(jlo / kPg);
+  for (int pg = jlo / kPg; pg <= pg_last; ++pg) {
+    const int kt = pg * kPg;
+    stash();
     __syncthreads();                                   // tiles visible
+    if (pg < pg_last) fetch(pg + 1);
     if (active) {
       f32x4 sc[2];
 #pragma unroll
@@ -160,8 +187,8 @@ __global__ __launch_bounds__(256, 2) void attn_mixq_mfma_kernel(
 #pragma unroll
       for (int m = 0; m < VT; ++m) {
         const int r0 = 4 * g4 + q4, r1 = 16 + 4 * g4 + q4;
-        const s16x4 a0 = ds_read_tr16(v_lds + r0 * VD + 16 * m + 4 * p4);
-        const s16x4 a1 = ds_read_tr16(v_lds + r1 * VD + 16 * m + 4 * p4);
+        const s16x4 a0 = ds_read_tr16(v_lds + r0 * VRS + 16 * m + 4 * p4);
+        const s16x4 a1 = ds_read_tr16(v_lds + r1 * VRS + 16 * m + 4 * p4);
         const s16x8 a = (s16x8){a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
         o[m] *= alpha;
         o[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(pb_hi), o[m], 0, 0, 0);
@@ -190,9 +217,9 @@ static void launch_one(const float* qn, const float* ts, const bf16_t* k, const 
                        int W, bf16_t* out, int64_t out_stride, const float* slopes,
                        const float* sink, int chunk, int H, int G, int dim, hipStream_t s) {
   const int rep = H / G;
-  const int nwaves = 2 * rep < 4 ? 2 * rep : 4;
+  const int nwaves = 4;                  // waves without a column tile still load the pages
   const int z = (2 * rep + nwaves - 1) / nwaves;
-  const size_t lds = ((size_t)kPg * (EK * 32 + kKPad) + (size_t)kPg * VT * 16) * sizeof(bf16_t);
+  const size_t lds = ((size_t)kPg * (EK * 32 + kKPad) + (size_t)kPg * (VT * 16 + kKPad)) * sizeof(bf16_t);
   static bool attr = false;
   if (!attr) {          // dynamic LDS above 64 KB has to be allowed per kernel, once
     hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mixq_mfma_kernel<EK, VT>),

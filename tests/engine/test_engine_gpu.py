@@ -100,6 +100,8 @@ def test_engine_generates_valid_rfq_json(gpu):
 def test_graph_replay_matches_eager_forward(gpu):
     """A captured decode forward replays to bit-identical logits (same kernels, same
     shapes) and picks up new metadata written into its static input buffers."""
+    from replisense_rfq_amd import ops
+
     ops.reset_plans()            # a bare model: no plan of an earlier engine applies
     cfg = get_config("tiny-llama")
     m = DecoderLM(cfg, gpu, seed=5)
