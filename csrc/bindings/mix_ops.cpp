@@ -32,7 +32,7 @@ bool launch_attn_mixq_prefill(bool, const float*, const void*, const void*, cons
 bool launch_attn_mixq_prefill_mfma(const float*, const float*, const void*, const void*, const int32_t*, int,
                                    const int32_t*, const int32_t*, const int32_t*, const int32_t*,
                                    const int32_t*, int, void*, int64_t, const float*, const float*,
-                                   int, int, int, int, int, int, hipStream_t);
+                                   int, int, int, int, int, int, bool, hipStream_t);
 bool mixq_mfma_ok(int, int, int, int, int);
 }  // namespace rfqmix
 
@@ -208,7 +208,8 @@ void attn_mixq_prefill(const Tensor& qmix, const Tensor& k_cache, const Tensor& 
 void attn_mix_mfma(const Tensor& qn, const Tensor& ts, const Tensor& k_cache, const Tensor& v_cache,
                    const Tensor& bt, const Tensor& q_start, const Tensor& q_len,
                    const Tensor& kv_len, const Tensor& work_seq, const Tensor& work_qblk,
-                   const Tensor& out, const Tensor& slopes, const OptT& sink, int64_t chunk) {
+                   const Tensor& out, const Tensor& slopes, const OptT& sink, int64_t chunk,
+                   bool grouped) {
   TORCH_CHECK(!act_f32(k_cache, "attn_mix_mfma k_cache"), "attn_mix_mfma: bf16 caches");
   TORCH_CHECK(qn.dim() == 3 && k_cache.dim() == 4 && v_cache.dim() == 4, "attn_mix_mfma: qn [T, H, dim]");
   const int H = (int)qn.size(1), G = (int)k_cache.size(1), dim = (int)k_cache.size(3);
@@ -230,7 +231,7 @@ void attn_mix_mfma(const Tensor& qn, const Tensor& ts, const Tensor& k_cache, co
       i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB), i32p(kv_len, "kv_len", NB),
       i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W), W, out.data_ptr(),
       out.stride(0), f32p(slopes, "slopes", H), optf(sink, "sink", H), (int)chunk, H, G, dim, vdim,
-      BS, stream());
+      BS, grouped, stream());
   TORCH_CHECK(ok, "attn_mix_mfma: no tile for these sizes");
 }
 
@@ -258,7 +259,7 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("head_norm_append(Tensor qkv, Tensor q_w, Tensor k_w, float eps, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, int H, int G, int dim, int vdim, Tensor(c!) qn, Tensor? ts, Tensor(d!)? qmix, int mix_from) -> ()");
   m.def("attn_talk_decode(Tensor qn, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor(a!) out, Tensor slopes, Tensor? talk, Tensor? sink, float scale, int chunk, int max_rows) -> ()");
   m.def("attn_mixq_prefill(Tensor qmix, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor slopes, Tensor? sink, int chunk, int qblk) -> ()");
-  m.def("attn_mix_mfma(Tensor qn, Tensor ts, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor slopes, Tensor? sink, int chunk) -> ()");
+  m.def("attn_mix_mfma(Tensor qn, Tensor ts, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor slopes, Tensor? sink, int chunk, bool grouped) -> ()");
   m.def("glu_clamped(Tensor gate_up, float limit, float alpha, Tensor(a!) out) -> ()");
   m.def("mixq_mfma_ok", &mixq_mfma_ok);
 }

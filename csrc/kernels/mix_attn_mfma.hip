@@ -30,7 +30,10 @@ constexpr int kKPad = 8;           // bf16 elements of padding per K / V row in 
                                    // of 16 B modulo 128 B, so the 8 lanes of a 16-byte read
                                    // phase (rows c .. c + 7) fall into different banks
 
-template <int EK, int VT>
+// GRP (decode section): the four waves of a workgroup take four key/value heads (one column
+// tile each) instead of four column tiles of one head, so the staged key page serves four
+// times the heads; every wave stages its own head's V tile.
+template <int EK, int VT, bool GRP>
 __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
     const float* __restrict__ qn, const float* __restrict__ ts, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int maxb,
@@ -42,19 +45,22 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
   constexpr int VD = VT * 16, E = EK * 32, RS = E + kKPad, VRS = VD + kKPad;
   extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
   bf16_t* k_lds = lds;                       // [32][RS]
-  bf16_t* v_lds = lds + kPg * RS;            // [32][VRS]
+  bf16_t* v_lds = lds + kPg * RS;            // [32][VRS], one per wave with GRP
   const int s = work_seq[blockIdx.x];
   if (s < 0) return;
   const int ql = q_len[s], kl = kv_len[s];
   const int i0 = work_qblk[blockIdx.x] * 32;
   if (i0 >= ql) return;
   const int nq = min(32, ql - i0);
-  const int cg = blockIdx.y, rep = H / G;
+  const int rep = H / G;
   const int nwaves = blockDim.x >> 6, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  if (blockIdx.z * nwaves * 16 >= nq * rep) return;     // no column of this workgroup is used
+  if ((GRP ? blockIdx.z : blockIdx.z * nwaves) * 16 >= nq * rep) return;   // no column is used
+  const int cg_raw = GRP ? blockIdx.y * 4 + wave : blockIdx.y;
+  const int cg = cg_raw < G ? cg_raw : 0;
   const int g4 = lane >> 4, c = lane & 15;
-  const int tile = blockIdx.z * nwaves + wave;
-  const bool active = tile * 16 < nq * rep;             // wave-uniform
+  const int tile = GRP ? blockIdx.z : blockIdx.z * nwaves + wave;
+  const bool active = cg_raw < G && tile * 16 < nq * rep;      // wave-uniform
+  if (GRP) v_lds += wave * kPg * VRS;
   const int col = tile * 16 + c;
   const int tok = col / rep, hh = cg * rep + col % rep;
   const bool cvalid = active && tok < nq;
@@ -94,7 +100,9 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
 
   // Page pipeline: the next page's K / V pieces are loaded into registers while this page is
   // multiplied out of LDS (one memory round trip per page, hidden behind the MFMAs).
-  constexpr int NK = (kPg * (E / 8) + 255) / 256, NV = (kPg * (VD / 8) + 255) / 256;
+  constexpr int NK = (kPg * (E / 8) + 255) / 256;
+  constexpr int VTHR = GRP ? 64 : 256, NV = (kPg * (VD / 8) + VTHR - 1) / VTHR;
+  const int vtid = GRP ? lane : threadIdx.x;
   s16x8 kreg[NK], vreg[NV];
   int kdst[NK];                                        // LDS element offset of every K piece
   {
@@ -115,7 +123,7 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
       if (kdst[u] >= 0) kreg[u] = kb[threadIdx.x + u * 256];
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      const int x = threadIdx.x + u * 256;
+      const int x = vtid + u * VTHR;
       // rows past the last written key are zeroed (they may hold anything, and 0 * NaN
       // would poison the sum)
       if (x < kPg * (VD / 8))
@@ -128,7 +136,7 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
       if (kdst[u] >= 0) *reinterpret_cast<s16x8*>(k_lds + kdst[u]) = kreg[u];
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      const int x = threadIdx.x + u * 256;
+      const int x = vtid + u * VTHR;
       if (x < kPg * (VD / 8))
         *reinterpret_cast<s16x8*>(v_lds + (x / (VD / 8)) * VRS + 8 * (x % (VD / 8))) = vreg[u];
     }
@@ -210,7 +218,7 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
   }
 }
 
-template <int EK, int VT>
+template <int EK, int VT, bool GRP>
 static void launch_one(const float* qn, const float* ts, const bf16_t* k, const bf16_t* v, const int32_t* bt,
                        int maxb, const int32_t* q_start, const int32_t* q_len,
                        const int32_t* kv_len, const int32_t* work_seq, const int32_t* work_qblk,
@@ -218,15 +226,17 @@ static void launch_one(const float* qn, const float* ts, const bf16_t* k, const 
                        const float* sink, int chunk, int H, int G, int dim, hipStream_t s) {
   const int rep = H / G;
   const int nwaves = 4;                  // waves without a column tile still load the pages
-  const int z = (2 * rep + nwaves - 1) / nwaves;
-  const size_t lds = ((size_t)kPg * (EK * 32 + kKPad) + (size_t)kPg * (VT * 16 + kKPad)) * sizeof(bf16_t);
+  const int z = GRP ? 2 * rep : (2 * rep + nwaves - 1) / nwaves;
+  const int gy = GRP ? (G + 3) / 4 : G;
+  const size_t lds = ((size_t)kPg * (EK * 32 + kKPad) +
+                      (size_t)(GRP ? 4 : 1) * kPg * (VT * 16 + kKPad)) * sizeof(bf16_t);
   static bool attr = false;
   if (!attr) {          // dynamic LDS above 64 KB has to be allowed per kernel, once
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mixq_mfma_kernel<EK, VT>),
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mixq_mfma_kernel<EK, VT, GRP>),
                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     attr = true;
   }
-  hipLaunchKernelGGL((attn_mixq_mfma_kernel<EK, VT>), dim3(W, G, z), dim3(nwaves * 64), lds, s, qn,
+  hipLaunchKernelGGL((attn_mixq_mfma_kernel<EK, VT, GRP>), dim3(W, gy, z), dim3(nwaves * 64), lds, s, qn,
                      ts, k, v, bt, maxb, q_start, q_len, kv_len, work_seq, work_qblk, out, out_stride,
                      slopes, sink, chunk, H, G, dim);
 }
@@ -246,15 +256,20 @@ bool launch_attn_mixq_prefill_mfma(const float* qn, const float* ts, const void*
                                    const int32_t* work_seq, const int32_t* work_qblk, int W,
                                    void* out, int64_t out_stride, const float* slopes,
                                    const float* sink, int chunk, int H, int G, int dim, int vdim,
-                                   int BS, hipStream_t s) {
+                                   int BS, bool grouped, hipStream_t s) {
   if (!mixq_mfma_ok(H, G, dim, vdim, BS)) return false;
   if (W == 0) return true;
   const int EK = G * dim / 32, VT = vdim / 16;
 #define MIXQ_CASE(ek, vt)                                                                       \
   if (EK == ek && VT == vt) {                                                                   \
-    launch_one<ek, vt>(qn, ts, (const bf16_t*)k_cache, (const bf16_t*)v_cache, bt, maxb, q_start, \
-                       q_len, kv_len, work_seq, work_qblk, W, (bf16_t*)out, out_stride, slopes, \
-                       sink, chunk, H, G, dim, s);                                              \
+    if (grouped)                                                                                \
+      launch_one<ek, vt, true>(qn, ts, (const bf16_t*)k_cache, (const bf16_t*)v_cache, bt, maxb, \
+                               q_start, q_len, kv_len, work_seq, work_qblk, W, (bf16_t*)out,   \
+                               out_stride, slopes, sink, chunk, H, G, dim, s);                 \
+    else                                                                                        \
+      launch_one<ek, vt, false>(qn, ts, (const bf16_t*)k_cache, (const bf16_t*)v_cache, bt, maxb, \
+                                q_start, q_len, kv_len, work_seq, work_qblk, W, (bf16_t*)out,  \
+                                out_stride, slopes, sink, chunk, H, G, dim, s);                \
     return true;                                                                                \
   }
   MIXQ_CASE(2, 2) MIXQ_CASE(2, 4) MIXQ_CASE(2, 8)

@@ -139,7 +139,8 @@ class LivisunLM:
                 ids, zeros = self._decode_work(m.dec_q_len.shape[0])
                 ops.attn_mix_mfma(qn[:D], lw["talk_scaled"], self.kv_k[li], self.kv_v[li],
                                   m.dec_block_tables, m.dec_q_start, m.dec_q_len, m.dec_kv_len,
-                                  ids, zeros, attn[:D], lw["slopes_mixed"], lw["sink"], mx.chunk)
+                                  ids, zeros, attn[:D], lw["slopes_mixed"], lw["sink"], mx.chunk,
+                                  grouped=True)
             elif D > 0:
                 ops.attn_talk_decode(qn[:D], self.kv_k[li], self.kv_v[li], m.dec_block_tables,
                                      m.dec_q_start, m.dec_q_len, m.dec_kv_len, attn[:D],

@@ -1103,13 +1103,14 @@ def attn_mixq_prefill(qmix, k_cache, v_cache, block_tables, q_start, q_len, kv_l
 
 
 def attn_mix_mfma(qn, talk_scaled, k_cache, v_cache, block_tables, q_start, q_len, kv_len,
-                  work_seq, work_qblk, out, slopes, sink, chunk: int):
+                  work_seq, work_qblk, out, slopes, sink, chunk: int, grouped: bool = False):
     """attn_mixq_prefill on MFMA tiles (bf16 caches, sizes of mixq_mfma_ok): the queries come
-    normed but unmixed, [T, H, dim]; the kernel mixes them in registers."""
+    normed but unmixed, [T, H, dim]; the kernel mixes them in registers.  ``grouped``: the
+    form for few rows per sequence (decode section), four key/value heads per workgroup."""
     if _gpu(qn):
         _native.mix_ops().attn_mix_mfma(qn, talk_scaled, k_cache, v_cache, block_tables, q_start,
                                         q_len, kv_len, work_seq, work_qblk, out, slopes, sink,
-                                        int(chunk))
+                                        int(chunk), bool(grouped))
     else:
         T, H, dim = qn.shape
         G = k_cache.shape[1]

@@ -29,6 +29,6 @@ def gpu():
 
 @pytest.fixture(scope="session")
 def reference_root():
-    if not os.path.isdir(REFERENCE):
-        pytest.skip("reference snapshot not mounted")
+    if not os.path.isdir(os.path.join(REFERENCE, "tests", "assets")):
+        pytest.skip("reference snapshot not mounted (or mounted empty)")
     return REFERENCE

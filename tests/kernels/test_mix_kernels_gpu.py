@@ -137,7 +137,7 @@ def test_attn_talk_decode(dt, H, G, dim, vdim, chunk, use_talk, use_sink):
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,dim,vdim,chunk", CASES + [(2, 2, 64, 64, 0), (8, 2, 128, 128, 96)])
-@pytest.mark.parametrize("mfma", [False, True])
+@pytest.mark.parametrize("mfma", [False, True, "grouped"])
 def test_attn_mixq_prefill(dt, H, G, dim, vdim, chunk, mfma):
     if mfma and dt != torch.bfloat16:
         pytest.skip("the MFMA tiles are bf16")
@@ -165,7 +165,7 @@ def test_attn_mixq_prefill(dt, H, G, dim, vdim, chunk, mfma):
     args = (kc.to(DEV), vc.to(DEV), m["bt"].to(DEV), m["q_start"].to(DEV), m["q_len"].to(DEV),
             m["kv_len"].to(DEV), ws.to(DEV), wq.to(DEV), got, slopes.to(DEV), sink.to(DEV), chunk)
     if mfma:
-        ops.attn_mix_mfma(qn.to(DEV), ts.to(DEV), *args)
+        ops.attn_mix_mfma(qn.to(DEV), ts.to(DEV), *args, grouped=mfma == "grouped")
     else:
         ops.attn_mixq_prefill(qmix.to(DEV), *args)
     torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
