@@ -41,24 +41,39 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
     const int32_t* __restrict__ kv_len, const int32_t* __restrict__ work_seq,
     const int32_t* __restrict__ work_qblk, bf16_t* __restrict__ out, int64_t out_stride,
     const float* __restrict__ slopes, const float* __restrict__ sink, int chunk, int H, int G,
-    int dim) {
+    int dim, int W, int nz) {
   constexpr int VD = VT * 16, E = EK * 32, RS = E + kKPad, VRS = VD + kKPad;
   extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
   bf16_t* k_lds = lds;                       // [32][RS]
   bf16_t* v_lds = lds + kPg * RS;            // [32][VRS], one per wave with GRP
-  const int s = work_seq[blockIdx.x];
+  // Work mapping.  GRP: grid (work item, group of four value heads, column tile).  Otherwise a
+  // 1-D grid that is XCD-aware: consecutive workgroups go to the 8 XCDs in turn, and each XCD
+  // has its own L2, so the G * nz workgroups of one work item (they all stream the same key
+  // pages) get ids 8 apart -- same XCD, launched back to back -- and read each page from HBM /
+  // MALL once and from that L2 otherwise.
+  int wi, by, bz;
+  if (GRP) {
+    wi = blockIdx.x; by = blockIdx.y; bz = blockIdx.z;
+  } else {
+    const int n = blockIdx.x, per = G * nz, k = n >> 3;
+    wi = (k / per) * 8 + (n & 7);
+    const int yz = k % per;
+    by = yz / nz; bz = yz - by * nz;
+    if (wi >= W) return;
+  }
+  const int s = work_seq[wi];
   if (s < 0) return;
   const int ql = q_len[s], kl = kv_len[s];
-  const int i0 = work_qblk[blockIdx.x] * 32;
+  const int i0 = work_qblk[wi] * 32;
   if (i0 >= ql) return;
   const int nq = min(32, ql - i0);
   const int rep = H / G;
   const int nwaves = blockDim.x >> 6, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  if ((GRP ? blockIdx.z : blockIdx.z * nwaves) * 16 >= nq * rep) return;   // no column is used
-  const int cg_raw = GRP ? blockIdx.y * 4 + wave : blockIdx.y;
+  if ((GRP ? bz : bz * nwaves) * 16 >= nq * rep) return;   // no column is used
+  const int cg_raw = GRP ? by * 4 + wave : by;
   const int cg = cg_raw < G ? cg_raw : 0;
   const int g4 = lane >> 4, c = lane & 15;
-  const int tile = GRP ? blockIdx.z : blockIdx.z * nwaves + wave;
+  const int tile = GRP ? bz : bz * nwaves + wave;
   const bool active = cg_raw < G && tile * 16 < nq * rep;      // wave-uniform
   if (GRP) v_lds += wave * kPg * VRS;
   const int col = tile * 16 + c;
@@ -71,24 +86,47 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
   const int32_t* bt = block_tables + (int64_t)s * maxb;
   const float slope = slopes[hh];
 
-  // mixed queries of this lane's column as B operands (k = 8 g4 + j of every 32-slice)
+  // mixed queries of this lane's column as B operands (k = 8 g4 + j of every 32-slice).  The
+  // loop over the heads of a group has a run-time length, so it is the middle loop: each of
+  // its rounds issues the loads of KB slices at once instead of one load per round trip.
   s16x8 qf[EK];
   {
+    constexpr int KB = EK < 8 ? EK : 8;
     const float* qt = qn + (int64_t)(q_start[s] + i0 + (cvalid ? tok : 0)) * H * dim;
     const float* tr = ts + (int64_t)hh * H;
 #pragma unroll
-    for (int ks = 0; ks < EK; ++ks) {
-      const int e0 = 32 * ks + 8 * g4, ck = e0 / dim, x0 = e0 - ck * dim;
-      float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int kg = 0; kg < EK; kg += KB) {
+      float f[KB][8];
+      int hq[KB], xo[KB];
+#pragma unroll
+      for (int k = 0; k < KB; ++k) {
+        const int e0 = 32 * (kg + k) + 8 * g4, ck = e0 / dim;
+        hq[k] = ck * rep;
+        xo[k] = e0 - ck * dim;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[k][j] = 0.f;
+      }
       if (cvalid)
         for (int r = 0; r < rep; ++r) {
-          const float w = tr[ck * rep + r];
-          const float4* q4p = reinterpret_cast<const float4*>(qt + (int64_t)(ck * rep + r) * dim + x0);
-          const float4 a = q4p[0], b = q4p[1];
-          f[0] += w * a.x; f[1] += w * a.y; f[2] += w * a.z; f[3] += w * a.w;
-          f[4] += w * b.x; f[5] += w * b.y; f[6] += w * b.z; f[7] += w * b.w;
+          float w[KB];
+          float4 a[KB], b[KB];
+#pragma unroll
+          for (int k = 0; k < KB; ++k) {
+            w[k] = tr[hq[k] + r];
+            const float4* q4p = reinterpret_cast<const float4*>(qt + (int64_t)(hq[k] + r) * dim + xo[k]);
+            a[k] = q4p[0];
+            b[k] = q4p[1];
+          }
+#pragma unroll
+          for (int k = 0; k < KB; ++k) {
+            f[k][0] += w[k] * a[k].x; f[k][1] += w[k] * a[k].y;
+            f[k][2] += w[k] * a[k].z; f[k][3] += w[k] * a[k].w;
+            f[k][4] += w[k] * b[k].x; f[k][5] += w[k] * b[k].y;
+            f[k][6] += w[k] * b[k].z; f[k][7] += w[k] * b[k].w;
+          }
         }
-      qf[ks] = pack8(f);
+#pragma unroll
+      for (int k = 0; k < KB; ++k) qf[kg + k] = pack8(f[k]);
     }
   }
   f32x4 o[VT];
@@ -260,9 +298,10 @@ static void launch_one(const float* qn, const float* ts, const bf16_t* k, const 
                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     attr = true;
   }
-  hipLaunchKernelGGL((attn_mixq_mfma_kernel<EK, VT, GRP>), dim3(W, gy, z), dim3(nwaves * 64), lds, s, qn,
+  const dim3 grid = GRP ? dim3(W, gy, z) : dim3(((W + 7) / 8) * 8 * G * z);
+  hipLaunchKernelGGL((attn_mixq_mfma_kernel<EK, VT, GRP>), grid, dim3(nwaves * 64), lds, s, qn,
                      ts, k, v, bt, maxb, q_start, q_len, kv_len, work_seq, work_qblk, out, out_stride,
-                     slopes, sink, chunk, H, G, dim);
+                     slopes, sink, chunk, H, G, dim, W, z);
 }
 
 // Sizes the MFMA tiles cover: 32-token pages, dim a multiple of 32, E = G dim in
