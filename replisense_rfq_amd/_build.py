@@ -191,6 +191,27 @@ def build_runtime(verbose: bool = False) -> Path:
     return RT_SO
 
 
+def _newer_than(so: Path, sources) -> bool:
+    """The library exists and no source of it was modified after it was linked."""
+    if not so.exists():
+        return False
+    t = so.stat().st_mtime
+    return all(Path(p).stat().st_mtime <= t for p in sources)
+
+
+def ensure_runtime() -> Path:
+    """``_runtime`` built if it is missing or older than its sources (a start-up check that
+    costs no compiler run when the tree is built)."""
+    srcs = list((CSRC / "runtime").glob("*.cpp")) + list((CSRC / "runtime").glob("*.h"))
+    return RT_SO if _newer_than(RT_SO, srcs) else build_runtime()
+
+
+def ensure_mix_kernels() -> Path:
+    srcs = list((CSRC / "kernels").glob("mix_*")) + [CSRC / "kernels" / "common.h",
+                                                     CSRC / "bindings" / "mix_ops.cpp"]
+    return MIX_SO if _newer_than(MIX_SO, srcs) else build_mix_kernels()
+
+
 def build_all(verbose: bool = True) -> None:
     build_runtime(verbose)
     build_kernels(verbose=verbose)
