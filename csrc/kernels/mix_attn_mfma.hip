@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
   const bool cvalid = active && tok < nq;
   const int p0 = kl - ql + i0, plast = p0 + nq - 1;
   const int pi = p0 + (cvalid ? tok : 0);
-  const int ci = chunk > 0 ? pi / chunk : 0;
+  const int klo = chunk > 0 ? (pi / chunk) * chunk : 0;      // first key of the query's block
   const int jlo = chunk > 0 ? (p0 / chunk) * chunk : 0;
   const int32_t* bt = block_tables + (int64_t)s * maxb;
   const float slope = slopes[hh];
@@ -211,15 +211,25 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
     __syncthreads();                                   // tiles visible
     if (PIPE && pg < pg_last) fetch(pg + 1);
     if (active) {
-      f32x4 sc[2];
+      // K fragments are read from LDS in batches of KF slices (both key halves) before the
+      // MFMAs that use them, so the LDS latency is paid once per batch and not per MFMA
+      constexpr int KF = EK < 8 ? EK : 8;
+      f32x4 sc[2] = {(f32x4){0.f, 0.f, 0.f, 0.f}, (f32x4){0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        sc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int k0 = 0; k0 < EK; k0 += KF) {
+        s16x8 kf[2][KF];
 #pragma unroll
-        for (int ks = 0; ks < EK; ++ks) {
-          const s16x8 kf = *reinterpret_cast<const s16x8*>(ka + 16 * mt * RS + 32 * ks);
-          sc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[ks]),
-                                                           sc[mt], 0, 0, 0);
+        for (int k = 0; k < KF; ++k) {
+          kf[0][k] = *reinterpret_cast<const s16x8*>(ka + 32 * (k0 + k));
+          kf[1][k] = *reinterpret_cast<const s16x8*>(ka + 16 * RS + 32 * (k0 + k));
+        }
+        __builtin_amdgcn_sched_barrier(0);             // keep the reads ahead of the MFMAs
+#pragma unroll
+        for (int k = 0; k < KF; ++k) {
+          sc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[0][k]), as_bf16x8(qf[k0 + k]),
+                                                          sc[0], 0, 0, 0);
+          sc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[1][k]), as_bf16x8(qf[k0 + k]),
+                                                          sc[1], 0, 0, 0);
         }
       }
       // lane holds S^T[key = kt + 16 mt + 4 g4 + i][column c]
@@ -229,7 +239,7 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = kt + 16 * mt + 4 * g4 + i;
-          const bool ok = cvalid && key <= pi && (chunk == 0 || key / chunk == ci);
+          const bool ok = cvalid && key <= pi && key >= klo;
           const float v = ok ? sc[mt][i] - slope * (float)(pi - key) : -INFINITY;
           sc[mt][i] = v;
           mx = fmaxf(mx, v);
