@@ -249,20 +249,26 @@ __global__ __launch_bounds__(256) void attn_mixq_mfma_kernel(
       const float m_new = fmaxf(m_run, mx);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
       const float alpha = __expf(m_run - m_use);
-      float psum = 0.f, ph[8], pl[8];
+      float psum = 0.f, p[8];
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
-        const float p = __expf(sc[jj >> 2][jj & 3] - m_use);
-        psum += p;
-        ph[jj] = bf2f(f2bf(p));
-        pl[jj] = p - ph[jj];
+        p[jj] = __expf(sc[jj >> 2][jj & 3] - m_use);
+        psum += p[jj];
       }
       psum += __shfl_xor(psum, 16, 64);
       psum += __shfl_xor(psum, 32, 64);
       l_run = l_run * alpha + psum;
       m_run = m_new;
-      // P^T as B operand: element j <-> key (j < 4 ? 4 g4 + j : 16 + 4 g4 + j - 4)
-      const s16x8 pb_hi = pack8(ph), pb_lo = pack8(pl);
+      // P^T as B operand: element j <-> key (j < 4 ? 4 g4 + j : 16 + 4 g4 + j - 4); hi = the
+      // bf16 rounding of p (hardware conversion, two values per instruction), lo = bf16(p - hi)
+      u32x4 hb, lb;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        hb[i] = pack_bf16x2(p[2 * i], p[2 * i + 1]);
+        lb[i] = pack_bf16x2(p[2 * i] - __uint_as_float(hb[i] << 16),
+                            p[2 * i + 1] - __uint_as_float(hb[i] & 0xffff0000u));
+      }
+      const s16x8 pb_hi = __builtin_bit_cast(s16x8, hb), pb_lo = __builtin_bit_cast(s16x8, lb);
       const int q4 = c >> 2, p4 = c & 3;
 #pragma unroll
       for (int m = 0; m < VT; ++m) {
