@@ -231,12 +231,12 @@ __global__ __launch_bounds__(256) void attn_mixq_prefill_kernel(
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
       const int i = ti + 16 * a, pi = p0 + i;
-      const int ci = chunk > 0 ? pi / chunk : 0;
+      const int klo = chunk > 0 ? (pi / chunk) * chunk : 0;   // first key of the query's block
       float mx = kNegInf;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const int j = jb + tj + 16 * k;
-        const bool ok = i < nq && j <= pi && (chunk == 0 || j / chunk == ci);
+        const bool ok = i < nq && j <= pi && j >= klo;
         sacc[a][k] = ok ? sacc[a][k] - slope * (float)(pi - j) : kNegInf;
         mx = fmaxf(mx, sacc[a][k]);
       }
