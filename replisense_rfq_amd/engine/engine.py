@@ -102,10 +102,11 @@ class LLMEngine:
                 weights = load_safetensors(self.cfg.weights_path, self.model_cfg, tp, self.device,
                                            moe_ep=self.cfg.moe_parallel == "ep")
         if model is None and self.layered:
-            from ..models.livisun import LivisunLM
+            from ..models import layered_model_class
 
-            model = LivisunLM(self.model_cfg, self.device, tp, seed=self.cfg.seed,
-                              weights=weights, dtype=self.dtype)
+            model = layered_model_class(self.model_cfg.architecture)(
+                self.model_cfg, self.device, tp, seed=self.cfg.seed, weights=weights,
+                dtype=self.dtype)
         self.model = model or DecoderLM(self.model_cfg, self.device, tp, seed=self.cfg.seed,
                                         weights=weights, moe_ep=self.cfg.moe_parallel == "ep")
         # the norm weights go into qkv / gate|up before anything copies those weights
@@ -119,7 +120,7 @@ class LLMEngine:
             # one state slot per sequence in flight; slot and pages are handed out together
             self.kv = LayeredKVCache(self.model_cfg, self._num_blocks(), self.device,
                                      num_slots=self.cfg.max_num_seqs, dtype=self.dtype)
-            self.model.attach_kv_cache(self.kv.k, self.kv.v, self.kv.state)
+            self.model.attach_kv_cache(self.kv.k, self.kv.v, self.kv.state, self.kv.layer_state)
         else:
             self.kv = KVCache(self.model_cfg, self.model.hkv, self._num_blocks(), self.device,
                               prefix_cache=self.cfg.prefix_cache)

@@ -49,12 +49,21 @@ class KVCache:
 
 
 class LayeredKVCache:
-    """Pools of a layer-list model: one K and one V pool per layer, each with the layer's
-    own head count and sizes (``[num_blocks, G, block, dim]`` / ``[..., vdim]``), all
-    indexed by the same block ids, plus the state pool of the input convolutions:
-    ``[L, 2 sublayers, 2 * slots, taps - 1, d]`` fp32.  A sequence owns one slot while it
-    runs (native core); the pool is double buffered, a step reads half ``gen & 1`` of the
-    slot and writes the other, so rows of one launch never read what the launch writes."""
+    """Pools of a layer-list model, all indexed by the block ids of the one block manager.
+
+    Per layer, by the kind of its mixer:
+      attention          one K and one V pool with the layer's own head count and sizes
+                         (``[num_blocks, G, block, dim]`` / ``[..., vdim]``);
+      latent_attention   one pool ``[num_blocks, 1, block, kv_rank]`` of cached latents that
+                         serves as keys and as values; a layer that reads another layer's
+                         latent holds that layer's pool (the same tensor);
+      wkv                no pages.
+    Per-sequence state lives in slots; a sequence owns one while it runs (native core).  Every
+    state pool is double buffered: a step reads half ``gen & 1`` of the slot and writes the
+    other, so rows of one launch never read what the launch writes.  ``state``: the input
+    convolutions' last inputs ``[L, 2 sublayers, 2 * slots, taps - 1, d]`` fp32;
+    ``layer_state[i]``: name -> ``[2 * slots, ...]`` fp32 for what ``cfg.state_shapes(i)``
+    lists (a wkv layer's matrices and its previous input row)."""
 
     def __init__(self, cfg, num_blocks: int, device, num_slots: int, block_size: int = 32,
                  dtype=torch.bfloat16, prefix_cache: bool = False):
@@ -63,14 +72,29 @@ class LayeredKVCache:
         self.num_blocks = num_blocks
         self.num_slots = num_slots
         mk = torch.zeros if torch.device(device).type != "cuda" else torch.empty
-        self.k = [mk((num_blocks, ly.mixer.kv_heads, block_size, ly.mixer.dim), dtype=dtype,
-                     device=device) for ly in cfg.layers]
-        self.v = [mk((num_blocks, ly.mixer.kv_heads, block_size, ly.mixer.vdim), dtype=dtype,
-                     device=device) for ly in cfg.layers]
-        self.state = torch.zeros((cfg.n_layers, 2, 2 * num_slots, max(0, cfg.canon_taps - 1),
-                                  cfg.hidden), dtype=torch.float32, device=device)
+        self.k, self.v = [], []
+        for ly in cfg.layers:
+            m = ly.mixer
+            if m.kind == "attention":
+                self.k.append(mk((num_blocks, m.kv_heads, block_size, m.dim), dtype=dtype, device=device))
+                self.v.append(mk((num_blocks, m.kv_heads, block_size, m.vdim), dtype=dtype, device=device))
+            elif m.kind == "latent_attention":
+                pool = self.k[m.kv_from] if m.kv_from >= 0 else \
+                    mk((num_blocks, 1, block_size, m.kv_rank), dtype=dtype, device=device)
+                self.k.append(pool)
+                self.v.append(pool)
+            else:
+                self.k.append(None)
+                self.v.append(None)
+        self.state = torch.zeros((cfg.n_layers if cfg.canon_taps > 0 else 0, 2, 2 * num_slots,
+                                  max(0, cfg.canon_taps - 1), cfg.hidden),
+                                 dtype=torch.float32, device=device)
+        self.layer_state = [{name: torch.zeros((2 * num_slots,) + tuple(shape), dtype=torch.float32,
+                                               device=device)
+                             for name, shape in cfg.state_shapes(i).items()}
+                            for i in range(cfg.n_layers)]
         self.scratch_block = num_blocks - 1
-        self.prefix_cache = False            # a cached page carries no convolution state
+        self.prefix_cache = False            # a cached page carries no per-sequence state
         self.core = None
 
     @staticmethod

@@ -1,0 +1,15 @@
+"""Model classes.  Layer-list models are chosen by their configuration's architecture."""
+
+
+def layered_model_class(architecture: str):
+    """Model class of a layer-list architecture (imported on demand: each brings only the
+    kernels it runs)."""
+    if architecture == "Livisun":
+        from .livisun import LivisunLM
+
+        return LivisunLM
+    if architecture == "Numalorn":
+        from .numalorn import NumalornLM
+
+        return NumalornLM
+    raise KeyError(f"no model class for architecture {architecture!r}")

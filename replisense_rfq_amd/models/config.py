@@ -88,9 +88,15 @@ def get_config(name: str) -> ModelConfig:
 # every layer owns its KV pool shape).  Livisun is the first of them.
 @dataclass(frozen=True)
 class MixerSpec:
-    """Attention mixer: H query heads over G key/value heads, per-head query/key
-    size ``dim`` and value size ``vdim``; scores are scaled by ``scale``; position
-    i sees j <= i inside its own block of ``chunk`` positions (0 = plain causal)."""
+    """A layer's token mixer.
+
+    ``attention``: H query heads over G key/value heads, per-head query/key size ``dim``
+    and value size ``vdim``; scores are scaled by ``scale``; position i sees j <= i inside
+    its own block of ``chunk`` positions (0 = plain causal).
+    ``latent_attention``: queries through a ``q_rank`` latent, keys and values are per-head
+    up-projections of one cached ``kv_rank`` latent per token; ``kv_from`` >= 0 names the
+    layer whose cached latent this layer reads instead of projecting its own.
+    ``wkv``: ``heads`` recurrent heads with a ``dim`` x ``dim`` state each (no cache pages)."""
     kind: str = "attention"
     heads: int = 4
     kv_heads: int = 2
@@ -98,6 +104,9 @@ class MixerSpec:
     vdim: int = 64
     scale: float = 0.125
     chunk: int = 0
+    q_rank: int = 0
+    kv_rank: int = 0
+    kv_from: int = -1
 
     @property
     def group(self) -> int:
@@ -106,9 +115,18 @@ class MixerSpec:
 
 @dataclass(frozen=True)
 class MlpSpec:
+    """``dense``: clamped GLU of width ``ff``.  ``moe``: ``experts`` SwiGLU experts of width
+    ``ff``, ``top`` per token, chosen among the ``keep`` best of ``groups`` equal groups of
+    neighbouring experts (groups = 0: no limit), plus a shared expert of width
+    ``shared_ff`` (0: none)."""
     kind: str = "dense"
     ff: int = 256
     limit: float = 7.0
+    experts: int = 0
+    top: int = 0
+    groups: int = 0
+    keep: int = 0
+    shared_ff: int = 0
 
 
 @dataclass(frozen=True)
@@ -132,6 +150,9 @@ class LayeredConfig:
     bos_id: int = 0
     eos_ids: tuple = ()
     n_experts: int = 0
+    residual_mult: float = 1.0      # Numalorn: x += residual_mult * norm(sublayer(x))
+    logit_softcap: float = 0.0      # > 0: logits <- cap * tanh(logits / cap)
+    decay_rank: int = 16            # wkv layers of seeded models (a checkpoint's shapes decide)
 
     @property
     def n_layers(self) -> int:
@@ -145,15 +166,38 @@ class LayeredConfig:
         d, n = self.hidden, 0
         for ly in self.layers:
             m = ly.mixer
-            n += d * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + m.heads * m.vdim * d
-            n += 2 * m.dim + m.heads * m.heads + m.heads + 6 * d + 2 * d * self.canon_taps
-            if ly.mlp is not None:
-                n += 3 * d * ly.mlp.ff
+            if m.kind == "attention":
+                n += d * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + m.heads * m.vdim * d
+                n += 2 * m.dim + m.heads * m.heads + m.heads + 6 * d + 2 * d * self.canon_taps
+            elif m.kind == "latent_attention":
+                n += d * m.q_rank + m.q_rank * m.heads * m.dim + m.heads * m.vdim * d
+                n += m.kv_rank * m.heads * (m.dim + m.vdim) + (d * m.kv_rank if m.kv_from < 0 else 0)
+            else:
+                n += 5 * d * m.heads * m.dim + 2 * d * self.decay_rank
+            f = ly.mlp
+            if f is not None and f.kind == "moe":
+                n += 3 * d * (f.ff * f.experts + f.shared_ff) + d * f.experts
+            elif f is not None:
+                n += 3 * d * f.ff
         return n + 2 * self.vocab_size * d + d
 
     def kv_bytes_per_token(self, tp: int = 1, dtype_bytes: int = 2) -> int:
-        return sum(ly.mixer.kv_heads * (ly.mixer.dim + ly.mixer.vdim) for ly in self.layers) \
-            * dtype_bytes
+        n = 0
+        for ly in self.layers:
+            m = ly.mixer
+            if m.kind == "attention":
+                n += m.kv_heads * (m.dim + m.vdim)
+            elif m.kind == "latent_attention" and m.kv_from < 0:
+                n += m.kv_rank
+        return max(1, n) * dtype_bytes
+
+    def state_shapes(self, li: int) -> dict:
+        """Per-sequence recurrent state of layer ``li`` besides cache pages and the input
+        convolutions: name -> shape of one slot (fp32)."""
+        m = self.layers[li].mixer
+        if m.kind == "wkv":
+            return {"wkv": (m.heads, m.dim, m.dim), "prev": (self.hidden,)}
+        return {}
 
     def to_dict(self):
         return asdict(self)
@@ -184,6 +228,71 @@ class LayeredConfig:
                    max_position=int(d.get("max_position", 8192)))
 
 
+def numalorn_from_json(d: dict, name: str | None = None) -> LayeredConfig:
+    """config.json of a Numalorn checkpoint: vocab, width, norm.eps, residual_mult,
+    logit_softcap and ``layers``: type ``latent_attention`` (heads, dim, vdim, q_rank,
+    kv_rank, scale, optional kv_from) or ``wkv`` (heads, dim), each with an ``mlp`` of kind
+    ``moe`` (expert.ff, router.experts / top / groups.count / groups.keep, shared.ff) or
+    null."""
+    layers = []
+    for i, ly in enumerate(d["layers"]):
+        m, kind = ly["mixer"], ly["type"]
+        if kind == "latent_attention":
+            src = m.get("kv_from")
+            mixer = MixerSpec(kind, int(m["heads"]), 1, int(m["dim"]), int(m["vdim"]),
+                              float(m["scale"]), 0, int(m["q_rank"]), int(m["kv_rank"]),
+                              -1 if src is None else int(src))
+            if mixer.kv_from >= 0:
+                if not 0 <= mixer.kv_from < i:
+                    raise ValueError(f"layer {i}: kv_from must name an earlier layer")
+                o = layers[mixer.kv_from].mixer
+                if o.kind != kind or o.kv_from >= 0 or o.kv_rank != mixer.kv_rank:
+                    raise ValueError(f"layer {i}: layer {mixer.kv_from} holds no latent of rank "
+                                     f"{mixer.kv_rank} of its own")
+        elif kind == "wkv":
+            mixer = MixerSpec(kind, int(m["heads"]), 0, int(m["dim"]), int(m["dim"]))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        f = ly.get("mlp")
+        mlp = None
+        if f is not None:
+            if f.get("kind") != "moe":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {f.get('kind')!r}")
+            r = f["router"]
+            g = r.get("groups") or {}
+            E, count = int(r["experts"]), int(g.get("count", 0))
+            if count and (E % count or not 0 < int(g["keep"]) <= count):
+                raise ValueError(f"layer {i}: {E} experts do not form {count} equal groups")
+            if count and int(r["top"]) > int(g["keep"]) * (E // count):
+                raise ValueError(f"layer {i}: the kept groups hold fewer than top experts")
+            mlp = MlpSpec("moe", int(f["expert"]["ff"]), 0.0, E, int(r["top"]), count,
+                          int(g.get("keep", 0)), int((f.get("shared") or {}).get("ff", 0)))
+        layers.append(LayerSpec(mixer, mlp))
+    return LayeredConfig(name=name or d["architecture"].lower(), architecture=d["architecture"],
+                         vocab_size=int(d["vocab"]), hidden=int(d["width"]), layers=tuple(layers),
+                         rms_eps=float(d["norm"]["eps"]), canon_taps=0,
+                         max_position=int(d.get("max_position", 8192)),
+                         residual_mult=float(d["residual_mult"]),
+                         logit_softcap=float(d.get("logit_softcap") or 0.0))
+
+
+def numalorn_layers(n, width_heads, dim, vdim, q_rank, kv_rank, wkv_heads, ff, experts, top,
+                    groups, keep, shared_ff, share_every=2, wkv_dim=64):
+    """n layers alternating latent attention and wkv; of every ``share_every`` attention
+    layers the later ones read the first attention layer's latent."""
+    out, first = [], -1
+    f = MlpSpec("moe", ff, 0.0, experts, top, groups, keep, shared_ff)
+    for i in range(n):
+        if i % 2 == 0:
+            src = first if first >= 0 and (i // 2) % share_every != 0 else -1
+            out.append(LayerSpec(MixerSpec("latent_attention", width_heads, 1, dim, vdim,
+                                           dim ** -0.5, 0, q_rank, kv_rank, src), f))
+            first = i if first < 0 else first
+        else:
+            out.append(LayerSpec(MixerSpec("wkv", wkv_heads, 0, wkv_dim, wkv_dim), f))
+    return tuple(out)
+
+
 def _livisun_layers(n, heads, kv_heads, dim, vdim, chunk, ff, scale=None, limit=7.0):
     m = MixerSpec("attention", heads, kv_heads, dim, vdim, scale or dim ** -0.5, chunk)
     return tuple(LayerSpec(m, MlpSpec("dense", ff, limit)) for _ in range(n))
@@ -194,10 +303,13 @@ TINY_LIVISUN = LayeredConfig("tiny-livisun", vocab_size=384, hidden=128, embed_s
                              layers=_livisun_layers(2, 6, 3, 32, 16, 24, 192, limit=1.5))
 LIVISUN_8B = LayeredConfig("livisun-8b", vocab_size=128256, hidden=4096, embed_scale=1.0,
                            layers=_livisun_layers(32, 32, 8, 128, 128, 2048, 14336))
-CONFIGS.update({c.name: c for c in (TINY_LIVISUN, LIVISUN_8B)})
+TINY_NUMALORN = LayeredConfig("tiny-numalorn", architecture="Numalorn", vocab_size=320, hidden=128,
+                              canon_taps=0, residual_mult=0.5, logit_softcap=20.0, decay_rank=8,
+                              layers=numalorn_layers(4, 4, 32, 16, 48, 64, 2, 64, 6, 2, 3, 2, 96))
+CONFIGS.update({c.name: c for c in (TINY_LIVISUN, LIVISUN_8B, TINY_NUMALORN)})
 
 # config.json "architecture" -> reader
-ARCHITECTURES = {"Livisun": LayeredConfig.from_json}
+ARCHITECTURES = {"Livisun": LayeredConfig.from_json, "Numalorn": numalorn_from_json}
 
 
 def load_config(path: str):

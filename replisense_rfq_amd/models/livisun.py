@@ -87,7 +87,7 @@ class LivisunLM:
     def tile_decode_weights(self, mode: str | None = None) -> int:
         return 0
 
-    def attach_kv_cache(self, k_pools, v_pools, state=None) -> None:
+    def attach_kv_cache(self, k_pools, v_pools, state=None, layer_state=None) -> None:
         """Per-layer pools [num_blocks, G, block, dim | vdim]; state [L, 2, 2*slots, taps-1, d]."""
         assert len(k_pools) == self.cfg.n_layers
         self.kv_k, self.kv_v, self.state = k_pools, v_pools, state

@@ -293,6 +293,8 @@ def load_layered_safetensors(path: str, cfg, device, dtype=torch.bfloat16) -> di
 
     files = sorted(glob.glob(os.path.join(path, "*.safetensors"))) if os.path.isdir(path) else [path]
     ck = _LazyCheckpoint(files)
+    if cfg.architecture == "Numalorn":
+        return _numalorn_assemble(ck.full, lambda k: k in ck, cfg, device, dtype)
     w = {"embed": ck.full("embed").to(dtype).to(device), "lm_head": ck.full("head").to(dtype).to(device),
          "final_norm": ck.full("final.norm").float().to(device), "vocab_start": 0, "layers": []}
     for i, ly in enumerate(cfg.layers):
@@ -351,4 +353,145 @@ def layered_from_full(full: dict, cfg, device, dtype=torch.bfloat16) -> dict:
         pre = f"l{i}."
         w["layers"].append(_assemble_layer(lambda k: full[pre + k], ly, lambda k: pre + k in full,
                                            dtype, device))
+    return w
+
+
+# --------------------------------------------------------------------------
+# Numalorn.  Checkpoint names:
+#   embed, head [V, d]; final.norm [d]; l<i>.norm1 | norm2 [d] (stored around zero)
+#   latent attention: l<i>.mix.dq [q_rank, d]  .dq.norm [q_rank]  .uq [H*dim, q_rank]
+#     .dkv [kv_rank, d]  .dkv.norm [kv_rank] (absent with kv_from)  .uk [H*dim, kv_rank]
+#     .uv [H*vdim, kv_rank]  .sink [H]  .o [d, H*vdim]
+#   wkv: l<i>.mix.mu.{r,k,v,g,w} [d]  .r | .k | .v | .g [H*N, d]  .w1 [rank, d]  .w2 [H*N, rank]
+#     .w0 [H*N]  .u [H, N]  .norm [H*N]  .o [d, H*N]
+#   moe: l<i>.mlp.router [E, d]  .correction [E]  .e<j>.gate | up [F, d]  .e<j>.down [d, F]
+#     .shared.gate | up [Fs, d]  .shared.down [d, Fs]
+# Loaded layout per layer: "down" = dq | dkv rows, uk [H, dim, R] and uv^T [H, R, vdim] for the
+# absorbed products, "rkvg" [4, H*N, d], w13 [E, 2F, d] gate | up rows, w2 [E, d, F]; norm
+# weights, mu, w0, u, sink, router and correction in fp32.
+def _numalorn_assemble(get, has, cfg, device, dtype) -> dict:
+    d = cfg.hidden
+
+    def mat(name, rows, cols):
+        t = get(name)
+        if tuple(t.shape) != (rows, cols):
+            raise ValueError(f"tensor {name}: shape {tuple(t.shape)}, expected {(rows, cols)}")
+        return t.to(dtype)
+
+    def vec(name, *shape):
+        t = get(name)
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"tensor {name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t.float().contiguous().to(device)
+
+    V = cfg.vocab_size
+    w = {"embed": mat("embed", V, d).to(device), "lm_head": mat("head", V, d).to(device),
+         "final_norm": vec("final.norm", d), "vocab_start": 0, "layers": []}
+    for i, ly in enumerate(cfg.layers):
+        p, m, lw = f"l{i}.", ly.mixer, LayerWeights()
+        lw["norm1"] = vec(p + "norm1", d)
+        if m.kind == "latent_attention":
+            H, R = m.heads, m.kv_rank
+            rows = [mat(p + "mix.dq", m.q_rank, d)]
+            if m.kv_from < 0:
+                rows.append(mat(p + "mix.dkv", R, d))
+                lw["dkv_norm"] = vec(p + "mix.dkv.norm", R)
+            lw["down"] = torch.cat(rows, 0).contiguous().to(device)
+            lw["dq_norm"] = vec(p + "mix.dq.norm", m.q_rank)
+            lw["uq"] = mat(p + "mix.uq", H * m.dim, m.q_rank).contiguous().to(device)
+            lw["uk"] = mat(p + "mix.uk", H * m.dim, R).view(H, m.dim, R).contiguous().to(device)
+            lw["uv_t"] = mat(p + "mix.uv", H * m.vdim, R).view(H, m.vdim, R).transpose(1, 2) \
+                .contiguous().to(device)
+            lw["sink"] = vec(p + "mix.sink", H)
+            lw["o"] = mat(p + "mix.o", d, H * m.vdim).contiguous().to(device)
+        else:
+            HN = m.heads * m.dim
+            lw["mu"] = torch.stack([vec(p + "mix.mu." + s, d) for s in "rkvgw"]).contiguous()
+            lw["rkvg"] = torch.stack([mat(p + "mix." + s, HN, d) for s in "rkvg"]).contiguous().to(device)
+            rank = get(p + "mix.w1").shape[0]
+            lw["w1"] = mat(p + "mix.w1", rank, d).contiguous().to(device)
+            lw["w2"] = mat(p + "mix.w2", HN, rank).contiguous().to(device)
+            lw["w0"] = vec(p + "mix.w0", HN)
+            lw["u"] = vec(p + "mix.u", m.heads, m.dim)
+            lw["gn"] = vec(p + "mix.norm", HN)
+            lw["o"] = mat(p + "mix.o", d, HN).contiguous().to(device)
+        f = ly.mlp
+        if f is not None:
+            q = p + "mlp."
+            lw["norm2"] = vec(p + "norm2", d)
+            lw["router"] = vec(q + "router", f.experts, d)
+            lw["correction"] = vec(q + "correction", f.experts)
+            lw["w13"] = torch.stack([torch.cat([mat(f"{q}e{e}.gate", f.ff, d), mat(f"{q}e{e}.up", f.ff, d)], 0)
+                                     for e in range(f.experts)]).contiguous().to(device)
+            lw["w2e"] = torch.stack([mat(f"{q}e{e}.down", d, f.ff) for e in range(f.experts)]) \
+                .contiguous().to(device)
+            if f.shared_ff:
+                lw["shared_gu"] = torch.cat([mat(q + "shared.gate", f.shared_ff, d),
+                                             mat(q + "shared.up", f.shared_ff, d)], 0).contiguous().to(device)
+                lw["shared_down"] = mat(q + "shared.down", d, f.shared_ff).contiguous().to(device)
+        w["layers"].append(lw)
+    return w
+
+
+def init_numalorn_weights(cfg, device, dtype=torch.bfloat16, seed: int = 0) -> dict:
+    """Seeded random Numalorn weights under the checkpoint's names (tests and benchmarks):
+    projections scaled so that activations stay O(1); sinks, corrections, bonuses, decays and
+    zero-centred norm weights away from their neutral values so that each shows in the logits."""
+    d, full = cfg.hidden, {}
+
+    def rnd(name, shape, std, mean=0.0):
+        t = _randn(shape, std, (seed, name), "cpu", torch.float32) + mean
+        full[name] = t.to(torch.bfloat16).float()
+        return full[name]
+
+    rnd("embed", (cfg.vocab_size, d), 1.0)
+    rnd("head", (cfg.vocab_size, d), 2.0 * d ** -0.5)
+    rnd("final.norm", (d,), 0.2)
+    for i, ly in enumerate(cfg.layers):
+        p, m = f"l{i}.", ly.mixer
+        rnd(p + "norm1", (d,), 0.2)
+        if m.kind == "latent_attention":
+            H, R = m.heads, m.kv_rank
+            rnd(p + "mix.dq", (m.q_rank, d), d ** -0.5)
+            rnd(p + "mix.dq.norm", (m.q_rank,), 0.1, 1.0)
+            rnd(p + "mix.uq", (H * m.dim, m.q_rank), 1.5 * m.q_rank ** -0.5)
+            if m.kv_from < 0:
+                rnd(p + "mix.dkv", (R, d), d ** -0.5)
+                rnd(p + "mix.dkv.norm", (R,), 0.1, 1.0)
+            rnd(p + "mix.uk", (H * m.dim, R), 1.5 * R ** -0.5)
+            rnd(p + "mix.uv", (H * m.vdim, R), R ** -0.5)
+            rnd(p + "mix.sink", (H,), 1.0)
+            rnd(p + "mix.o", (d, H * m.vdim), (H * m.vdim) ** -0.5)
+        else:
+            HN = m.heads * m.dim
+            for s in "rkvgw":
+                rnd(p + "mix.mu." + s, (d,), 0.25, 0.5)
+            for s in "rkvg":
+                rnd(p + "mix." + s, (HN, d), d ** -0.5)
+            rnd(p + "mix.w1", (cfg.decay_rank, d), d ** -0.5)
+            rnd(p + "mix.w2", (HN, cfg.decay_rank), cfg.decay_rank ** -0.5)
+            rnd(p + "mix.w0", (HN,), 1.0, -2.0)
+            rnd(p + "mix.u", (m.heads, m.dim), 0.5)
+            rnd(p + "mix.norm", (HN,), 0.1, 1.0)
+            rnd(p + "mix.o", (d, HN), HN ** -0.5)
+        f = ly.mlp
+        if f is not None:
+            q = p + "mlp."
+            rnd(p + "norm2", (d,), 0.2)
+            rnd(q + "router", (f.experts, d), 2.0 * d ** -0.5)
+            rnd(q + "correction", (f.experts,), 0.3)
+            for e in range(f.experts):
+                rnd(f"{q}e{e}.gate", (f.ff, d), d ** -0.5)
+                rnd(f"{q}e{e}.up", (f.ff, d), d ** -0.5)
+                rnd(f"{q}e{e}.down", (d, f.ff), f.ff ** -0.5)
+            if f.shared_ff:
+                rnd(q + "shared.gate", (f.shared_ff, d), d ** -0.5)
+                rnd(q + "shared.up", (f.shared_ff, d), d ** -0.5)
+                rnd(q + "shared.down", (d, f.shared_ff), f.shared_ff ** -0.5)
+    return numalorn_from_full(full, cfg, device, dtype)
+
+
+def numalorn_from_full(full: dict, cfg, device, dtype=torch.bfloat16) -> dict:
+    w = _numalorn_assemble(lambda k: full[k], lambda k: k in full, cfg, device, dtype)
+    w["full"] = full
     return w

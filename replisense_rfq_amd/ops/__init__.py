@@ -1134,3 +1134,123 @@ def glu_clamped(gate_up, limit: float, alpha: float = 1.702, out=None):
     else:
         ref.glu_clamped(gate_up, limit, alpha, out)
     return out
+
+
+# ---------------------------------------------------------------------------
+# Post-norm residual layers, latent attention, the wkv recurrence and grouped sigmoid
+# routing (csrc/kernels/mix_latent.hip, mix_wkv.hip, mix_route.hip; same library).
+_BMM_OUT_DTYPE = None
+
+
+def bmm_f32(a, b):
+    """Batched a[B, M, K] . b[B, K, N] on the vendor library with an fp32 result (the
+    accumulator's precision is kept for bf16 operands)."""
+    if a.dtype == torch.float32:
+        return torch.bmm(a, b)
+    global _BMM_OUT_DTYPE
+    if a.is_cuda and a.shape[1] > 0 and _BMM_OUT_DTYPE is not False:
+        if _BMM_OUT_DTYPE:
+            return torch.bmm(a, b, out_dtype=torch.float32)
+        try:                                   # first call (never inside a graph capture)
+            y = torch.bmm(a, b, out_dtype=torch.float32)
+            _BMM_OUT_DTYPE = True
+            return y
+        except (TypeError, RuntimeError):
+            _BMM_OUT_DTYPE = False
+    return torch.bmm(a.float(), b.float())
+
+
+def embed_rows(ids, table, out=None):
+    out = torch.empty((ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device) \
+        if out is None else out
+    if _gpu(table):
+        _native.mix_ops().embed_rows(ids, table, out)
+    else:
+        ref.embed_rows(ids, table, out)
+    return out
+
+
+def post_norm_add(y, residual, w, mult: float, eps: float, out=None):
+    """residual (fp32, in place) += mult * rms(y) * (1 + w); ``out`` (the model's dtype)
+    receives a copy of the updated stream for the next sublayer's products."""
+    if _gpu(residual):
+        _native.mix_ops().post_norm_add(y, residual, w, float(mult), float(eps), out)
+    else:
+        ref.post_norm_add(y, residual, w, mult, eps, out)
+    return out
+
+
+def rms_norm_rows(x, w, eps: float, out, offset: float = 0.0):
+    """out = rms(x) * (w + offset) per row in fp32; x may be a column slice of a wider
+    matrix."""
+    if _gpu(x):
+        _native.mix_ops().rms_norm_rows(x, w, float(eps), float(offset), out)
+    else:
+        ref.rms_norm_rows(x, w, eps, out, offset)
+    return out
+
+
+def latent_norm_append(x, w, eps: float, slot_mapping, pool):
+    if _gpu(x):
+        _native.mix_ops().latent_norm_append(x, w, float(eps), slot_mapping, pool)
+    else:
+        ref.latent_norm_append(x, w, eps, slot_mapping, pool)
+
+
+def token_shift_mix(x, mu, prev, row_state, row_back, row_fwd, positions, out):
+    if _gpu(x):
+        _native.mix_ops().token_shift_mix(x, mu, prev, row_state, row_back, row_fwd, positions, out)
+    else:
+        ref.token_shift_mix(x, mu, prev, row_state, row_back, row_fwd, positions, out)
+    return out
+
+
+def wkv_recurrence(r, k, v, zw, w0, u, gate, norm_w, eps: float, state, row_state, row_back,
+                   row_fwd, positions, out):
+    if _gpu(r):
+        _native.mix_ops().wkv_recurrence(r, k, v, zw, w0, u, gate, norm_w, float(eps), state,
+                                         row_state, row_back, row_fwd, positions, out)
+    else:
+        ref.wkv_recurrence(r, k, v, zw, w0, u, gate, norm_w, eps, state, row_state, row_back,
+                           row_fwd, positions, out)
+    return out
+
+
+def moe_route_grouped(z, correction, top: int, groups: int, keep: int, ids, weights):
+    if _gpu(z):
+        _native.mix_ops().moe_route_grouped(z, correction, int(top), int(groups), int(keep), ids,
+                                            weights)
+    else:
+        ref.moe_route_grouped(z, correction, top, groups, keep, ids, weights)
+
+
+def moe_experts(h, ids, weights, w13, w2, base, out):
+    """Routed experts of any sizes in either dtype, one (token, choice) pair per workgroup
+    row block; the weighted sum and ``base`` (the shared expert's output) add up in fp32."""
+    if _gpu(h):
+        F = w2.shape[2]
+        act = torch.empty((ids.numel(), F), dtype=h.dtype, device=h.device)
+        _native.mix_ops().moe_pair_up(h, ids, w13, act)
+        _native.mix_ops().moe_pair_down(act, ids, weights, w2, base, out)
+    else:
+        ref.moe_experts(h, ids, weights, w13, w2, base, out)
+    return out
+
+
+def silu_mul_any(gate_up, out=None):
+    F = gate_up.shape[1] // 2
+    out = torch.empty((gate_up.shape[0], F), dtype=gate_up.dtype, device=gate_up.device) \
+        if out is None else out
+    if _gpu(gate_up):
+        _native.mix_ops().silu_mul_any(gate_up, out)
+    else:
+        ref.silu_mul_any(gate_up, out)
+    return out
+
+
+def softcap(x, cap: float):
+    if _gpu(x):
+        _native.mix_ops().softcap(x, float(cap))
+    else:
+        ref.softcap(x, cap)
+    return x

@@ -353,3 +353,153 @@ def glu_clamped(gate_up, limit: float, alpha: float, out) -> None:
     g = gate_up[:, :F].float().clamp(max=limit)
     u = gate_up[:, F:].float().clamp(-limit, limit)
     out.copy_((g * torch.sigmoid(alpha * g) * (u + 1)).to(out.dtype))
+
+
+# --------------------------------------------------------------------------
+# Post-norm residual layers, latent attention, wkv recurrence, grouped sigmoid routing.
+def embed_rows(ids, table, out) -> None:
+    """out[t] = table[ids[t]] in fp32."""
+    out.copy_(table[ids.long()].float())
+
+
+def post_norm_add(y, residual, w, mult: float, eps: float, out) -> None:
+    """residual (fp32, in place) += mult * rms(y) * (1 + w); out (any dtype, may be None)
+    receives the updated residual: the next sublayer reads the stream itself."""
+    residual.add_(_rms(y.float(), eps) * (1.0 + w.float()) * mult)
+    if out is not None:
+        out.copy_(residual.to(out.dtype))
+
+
+def rms_norm_rows(x, w, eps: float, out, offset: float = 0.0) -> None:
+    """out = rms(x) * (w + offset) per row, computed in fp32; x may be a column slice."""
+    out.copy_((_rms(x.float(), eps) * (w.float() + offset)).to(out.dtype))
+
+
+def latent_norm_append(x, w, eps: float, slot_mapping, pool) -> None:
+    """c = rms(x) * w per row (fp32) into the paged latent pool [blocks, 1, BS, R] at the
+    rows' slots (slot < 0: dropped)."""
+    T = x.shape[0]
+    if T == 0:
+        return
+    BS = pool.shape[2]
+    c = _rms(x.float(), eps) * w.float()
+    slots = slot_mapping[:T].long()
+    ok = slots >= 0
+    if ok.any():
+        sl = slots[ok]
+        pool[sl // BS, 0, sl % BS] = c[ok].to(pool.dtype)
+
+
+def _state_rows(code: int, S: int):
+    """(read row, write row) of a state pool [2 * S, ...] for row_state code slot*2+half."""
+    return (code & 1) * S + (code >> 1), (1 - (code & 1)) * S + (code >> 1)
+
+
+def token_shift_mix(x, mu, prev, row_state, row_back, row_fwd, positions, out) -> None:
+    """out[s, t] = x[t] + (x'[t] - x[t]) * mu[s] for each of the mu rows, x' the previous
+    token's row of the same sequence: the row above inside a scheduled run, the sequence's
+    state half (prev [2 * slots, d] fp32) at the run's start, zeros at position 0.  The
+    run's last row goes to the other half."""
+    T, d = x.shape
+    if T == 0:
+        return
+    S = prev.shape[0] // 2
+    xf = x.float()
+    before = torch.zeros_like(xf)
+    new = []
+    for t in range(T):
+        code, i, f, p = int(row_state[t]), int(row_back[t]), int(row_fwd[t]), int(positions[t])
+        if i > 0:
+            before[t] = xf[t - 1]
+        elif p > 0 and code >= 0:
+            before[t] = prev[_state_rows(code, S)[0]]
+        if f == 0 and code >= 0:
+            new.append((_state_rows(code, S)[1], xf[t].clone()))
+    for wr, v in new:
+        prev[wr] = v
+    out.copy_((xf[None] + (before - xf)[None] * mu.float()[:, None, :]).to(out.dtype))
+
+
+def wkv_recurrence(r, k, v, zw, w0, u, gate, norm_w, eps: float, state, row_state, row_back,
+                   row_fwd, positions, out) -> None:
+    """Per head (N key x N value channels), token by token inside each scheduled run:
+        w_t = exp(-exp(zw_t + w0));  o_t = (S + diag(u) k_t v_t^T)^T r_t;  S <- diag(w_t) S + k_t v_t^T
+    then out_t = o_t / rms_head(o_t) * norm_w * silu(gate_t).  state: [2 * slots, H, N, N]
+    fp32, read from the row's half at the run's start (zeros at position 0), the run's last
+    state written to the other half.  Decay, state and output norm in fp32."""
+    T = r.shape[0]
+    if T == 0:
+        return
+    H, N = u.shape
+    S_ = state.shape[0] // 2
+    rf, kf, vf = (a.float().reshape(T, H, N) for a in (r, k, v))
+    w = torch.exp(-torch.exp(zw.float() + w0.float())).reshape(T, H, N)
+    uf = u.float()
+    o = torch.zeros(T, H, N)
+    cur = None
+    for t in range(T):
+        code, i, f, p = int(row_state[t]), int(row_back[t]), int(row_fwd[t]), int(positions[t])
+        if i == 0:
+            cur = state[_state_rows(code, S_)[0]].clone() if p > 0 and code >= 0 \
+                else torch.zeros(H, N, N)
+        kv = kf[t][:, :, None] * vf[t][:, None, :]
+        o[t] = torch.einsum("hkv,hk->hv", cur + uf[:, :, None] * kv, rf[t])
+        cur = w[t][:, :, None] * cur + kv
+        if f == 0 and code >= 0:
+            state[_state_rows(code, S_)[1]] = cur
+    y = _rms(o, eps).reshape(T, H * N) * norm_w.float() * torch.nn.functional.silu(gate.float())
+    out.copy_(y.to(out.dtype))
+
+
+def moe_route_grouped(z, correction, top: int, groups: int, keep: int, ids, weights) -> None:
+    """Sigmoid routing: s = sigmoid(z); experts are chosen by s + correction, only inside the
+    ``keep`` groups (of ``groups`` equal groups of neighbours; 0 = no limit) whose two largest
+    choice scores sum highest; weights = s of the chosen / (their sum + 1e-20).  Ties go to the
+    lower index."""
+    T, E = z.shape
+    s = torch.sigmoid(z.float())
+    choice = s + correction.float()
+    if groups > 0:
+        per = E // groups
+        grp = choice.view(T, groups, per)
+        gs = grp.topk(min(2, per), -1).values.sum(-1)
+        kept = torch.zeros(T, groups, dtype=torch.bool)
+        order = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep]
+        kept.scatter_(1, order, True)
+        choice = torch.where(kept[:, :, None].expand(T, groups, per), grp,
+                             torch.full_like(grp, float("-inf"))).reshape(T, E)
+    idx = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+    wt = s.gather(1, idx)
+    ids.copy_(idx.to(ids.dtype))
+    weights.copy_(wt / (wt.sum(-1, keepdim=True) + 1e-20))
+
+
+def silu_mul_any(gate_up, out) -> None:
+    """out = silu(gate) * up for gate_up = [gate | up] columns, any dtype and width."""
+    F = out.shape[1]
+    out.copy_((torch.nn.functional.silu(gate_up[:, :F].float()) * gate_up[:, F:].float()).to(out.dtype))
+
+
+def softcap(x, cap: float) -> None:
+    """x <- cap * tanh(x / cap), in place (fp32)."""
+    x.copy_(cap * torch.tanh(x / cap))
+
+
+def moe_experts(h, ids, weights, w13, w2, base, out) -> None:
+    """out (fp32) = base + sum_k weights[t, k] * W2[e] (silu(Wg[e] h_t) * (Wu[e] h_t)) with
+    e = ids[t, k]; w13 [E, 2F, d] holds gate | up rows, w2 [E, d, F].  Products in h's dtype
+    with fp32 accumulation, the weighted sum in fp32."""
+    T, F = h.shape[0], w2.shape[2]
+    acc = torch.zeros((T, w2.shape[1]), dtype=torch.float32) if base is None else base.float().clone()
+    for e in range(w13.shape[0]):
+        hit = (ids == e)
+        rows = hit.any(-1).nonzero()[:, 0]
+        if rows.numel() == 0:
+            continue
+        x = h[rows]
+        gu = x @ w13[e].t()
+        a = (torch.nn.functional.silu(gu[:, :F].float()) * gu[:, F:].float()).to(h.dtype)
+        y = (a @ w2[e].t()).float()
+        wt = (weights[rows] * hit[rows]).sum(-1)
+        acc[rows] += wt[:, None] * y
+    out.copy_(acc)
