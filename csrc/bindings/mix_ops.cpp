@@ -34,6 +34,29 @@ bool launch_attn_mixq_prefill_mfma(const float*, const float*, const void*, cons
                                    const int32_t*, int, void*, int64_t, const float*, const float*,
                                    int, int, int, int, int, int, bool, hipStream_t);
 bool mixq_mfma_ok(int, int, int, int, int);
+void launch_embed_rows(bool, const int32_t*, const void*, float*, int, int, int, hipStream_t);
+void launch_post_norm_add(bool, const void*, int64_t, float*, const float*, float, float, void*,
+                          int, int, hipStream_t);
+void launch_rms_norm_rows(bool, bool, const void*, int64_t, const float*, float, float, void*, int,
+                          int, hipStream_t);
+void launch_latent_norm_append(bool, const void*, int64_t, const float*, float, const int32_t*,
+                               void*, int, int, int64_t, hipStream_t);
+void launch_silu_mul_any(bool, const void*, int64_t, void*, int, int, hipStream_t);
+void launch_softcap(float*, float, int64_t, hipStream_t);
+void launch_token_shift_mix(bool, const float*, const float*, float*, const int32_t*,
+                            const int32_t*, const int32_t*, const int32_t*, void*, int, int, int,
+                            int, hipStream_t);
+bool wkv_ok(int);
+void launch_wkv_recurrence(bool, const void*, const void*, const void*, const void*, const void*,
+                           int64_t, int64_t, int64_t, int64_t, int64_t, const float*, const float*,
+                           const float*, float, float*, const int32_t*, const int32_t*,
+                           const int32_t*, const int32_t*, void*, int, int, int, int, hipStream_t);
+void launch_moe_route_grouped(const float*, const float*, int, int, int, int, int, int32_t*, float*,
+                              hipStream_t);
+void launch_moe_pair_up(bool, const void*, int64_t, const int32_t*, const void*, void*, int, int,
+                        int, int, int, hipStream_t);
+void launch_moe_pair_down(bool, const void*, const int32_t*, const float*, const void*, const void*,
+                          int64_t, float*, int, int, int, int, int, hipStream_t);
 }  // namespace rfqmix
 
 namespace {
@@ -250,6 +273,168 @@ void glu_clamped(const Tensor& gu, double limit, double alpha, const Tensor& out
                              (float)limit, (float)alpha, stream());
 }
 
+
+// ---- post-norm residual layers, latent norm, wkv, grouped sigmoid routing ----
+bool rows2d(const Tensor& t, int64_t T, int64_t n) {
+  return t.dim() == 2 && t.size(0) == T && t.size(1) == n && t.stride(1) == 1;
+}
+
+void embed_rows(const Tensor& ids, const Tensor& table, const Tensor& out) {
+  const bool f32 = act_f32(table, "embed_rows table");
+  const int T = (int)ids.numel(), d = (int)table.size(1);
+  TORCH_CHECK(table.dim() == 2 && table.is_contiguous(), "embed_rows: table [V, d]");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == d, "embed_rows: out [T, d]");
+  rfqmix::launch_embed_rows(f32, i32p(ids, "ids", T), table.data_ptr(),
+                            const_cast<float*>(f32p(out, "out")), T, d, (int)table.size(0), stream());
+}
+
+void post_norm_add(const Tensor& y, const Tensor& residual, const Tensor& w, double mult, double eps,
+                   const OptT& copy) {
+  const bool f32 = act_f32(y, "post_norm_add y");
+  TORCH_CHECK(residual.dim() == 2, "post_norm_add: residual [T, d]");
+  const int T = (int)residual.size(0), d = (int)residual.size(1);
+  TORCH_CHECK(rows2d(y, T, d), "post_norm_add: y [T, d]");
+  void* cp = nullptr;
+  if (copy.has_value()) {
+    TORCH_CHECK(copy->is_cuda() && copy->scalar_type() == at::kBFloat16 && copy->is_contiguous() &&
+                rows2d(*copy, T, d), "post_norm_add: copy [T, d] bfloat16");
+    cp = copy->data_ptr();
+  }
+  rfqmix::launch_post_norm_add(f32, y.data_ptr(), y.stride(0),
+                               const_cast<float*>(f32p(residual, "residual")), f32p(w, "w", d),
+                               (float)mult, (float)eps, cp, T, d, stream());
+}
+
+void rms_norm_rows(const Tensor& x, const Tensor& w, double eps, double offset, const Tensor& out) {
+  const bool fi = act_f32(x, "rms_norm_rows x"), fo = act_f32(out, "rms_norm_rows out");
+  TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1, "rms_norm_rows: x [T, n]");
+  const int T = (int)x.size(0), n = (int)x.size(1);
+  TORCH_CHECK(rows2d(out, T, n) && out.is_contiguous(), "rms_norm_rows: out [T, n]");
+  rfqmix::launch_rms_norm_rows(fi, fo, x.data_ptr(), x.stride(0), f32p(w, "w", n), (float)eps,
+                               (float)offset, out.data_ptr(), T, n, stream());
+}
+
+void latent_norm_append(const Tensor& x, const Tensor& w, double eps, const Tensor& slots,
+                        const Tensor& pool) {
+  const bool f32 = act_f32(x, "latent_norm_append x");
+  TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1, "latent_norm_append: x [T, R]");
+  const int T = (int)x.size(0), R = (int)x.size(1);
+  TORCH_CHECK(pool.is_cuda() && pool.dim() == 4 && pool.is_contiguous() && pool.size(1) == 1 &&
+              pool.size(3) == R && pool.scalar_type() == x.scalar_type(),
+              "latent_norm_append: pool [blocks, 1, BS, R] of x's dtype");
+  rfqmix::launch_latent_norm_append(f32, x.data_ptr(), x.stride(0), f32p(w, "w", R), (float)eps,
+                                    i32p(slots, "slot_mapping", T), pool.data_ptr(), T, R,
+                                    pool.size(0) * pool.size(2), stream());
+}
+
+void silu_mul_any(const Tensor& gu, const Tensor& out) {
+  const bool f32 = act_f32(gu, "silu_mul_any gate_up");
+  const int T = (int)gu.size(0), F = (int)out.size(1);
+  TORCH_CHECK(gu.dim() == 2 && gu.size(1) == 2 * F && gu.stride(1) == 1 && rows2d(out, T, F) &&
+              out.is_contiguous() && out.scalar_type() == gu.scalar_type(),
+              "silu_mul_any: gate_up [T, 2F], out [T, F]");
+  rfqmix::launch_silu_mul_any(f32, gu.data_ptr(), gu.stride(0), out.data_ptr(), T, F, stream());
+}
+
+void softcap(const Tensor& x, double cap) {
+  TORCH_CHECK(cap > 0, "softcap: cap > 0");
+  rfqmix::launch_softcap(const_cast<float*>(f32p(x, "logits")), (float)cap, x.numel(), stream());
+}
+
+void token_shift_mix(const Tensor& x, const Tensor& mu, const Tensor& prev, const Tensor& row_state,
+                     const Tensor& row_back, const Tensor& row_fwd, const Tensor& pos,
+                     const Tensor& out) {
+  TORCH_CHECK(x.dim() == 2 && mu.dim() == 2 && prev.dim() == 2, "token_shift_mix: x [T, d], mu [S, d], prev [2 slots, d]");
+  const int T = (int)x.size(0), d = (int)x.size(1), NS = (int)mu.size(0);
+  TORCH_CHECK(mu.size(1) == d && prev.size(1) == d && prev.size(0) % 2 == 0, "token_shift_mix: widths");
+  const bool fo = act_f32(out, "token_shift_mix out");
+  TORCH_CHECK(out.dim() == 3 && out.is_contiguous() && out.size(0) == NS && out.size(1) == T &&
+              out.size(2) == d, "token_shift_mix: out [S, T, d]");
+  rfqmix::launch_token_shift_mix(fo, f32p(x, "x"), f32p(mu, "mu"),
+                                 const_cast<float*>(f32p(prev, "prev")),
+                                 i32p(row_state, "row_state", T), i32p(row_back, "row_back", T),
+                                 i32p(row_fwd, "row_fwd", T), i32p(pos, "positions", T),
+                                 out.data_ptr(), T, d, NS, (int)prev.size(0) / 2, stream());
+}
+
+void wkv_recurrence(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& zw,
+                    const Tensor& w0, const Tensor& u, const Tensor& gate, const Tensor& norm_w,
+                    double eps, const Tensor& state, const Tensor& row_state,
+                    const Tensor& row_back, const Tensor& row_fwd, const Tensor& pos,
+                    const Tensor& out) {
+  const bool f32 = act_f32(r, "wkv_recurrence r");
+  TORCH_CHECK(u.dim() == 2, "wkv_recurrence: u [H, N]");
+  const int H = (int)u.size(0), N = (int)u.size(1), T = (int)r.size(0);
+  const int64_t HN = (int64_t)H * N;
+  for (const Tensor* t : {&r, &k, &v, &zw, &gate})
+    TORCH_CHECK(t->is_cuda() && rows2d(*t, T, HN) && t->scalar_type() == r.scalar_type(),
+                "wkv_recurrence: r, k, v, zw, gate [T, H N] of one dtype");
+  TORCH_CHECK(rows2d(out, T, HN) && out.is_contiguous() && out.scalar_type() == r.scalar_type(),
+              "wkv_recurrence: out [T, H N]");
+  TORCH_CHECK(state.dim() == 4 && state.size(0) % 2 == 0 && state.size(1) == H &&
+              state.size(2) == N && state.size(3) == N, "wkv_recurrence: state [2 slots, H, N, N]");
+  TORCH_CHECK(rfqmix::wkv_ok(N) && H <= 65535, "wkv_recurrence: head size outside the kernel's range");
+  rfqmix::launch_wkv_recurrence(
+      f32, r.data_ptr(), k.data_ptr(), v.data_ptr(), zw.data_ptr(), gate.data_ptr(), r.stride(0),
+      k.stride(0), v.stride(0), zw.stride(0), gate.stride(0), f32p(w0, "w0", HN), f32p(u, "u", HN),
+      f32p(norm_w, "norm_w", HN), (float)eps, const_cast<float*>(f32p(state, "state")),
+      i32p(row_state, "row_state", T), i32p(row_back, "row_back", T), i32p(row_fwd, "row_fwd", T),
+      i32p(pos, "positions", T), out.data_ptr(), T, H, N, (int)state.size(0) / 2, stream());
+}
+
+void moe_route_grouped(const Tensor& z, const Tensor& corr, int64_t top, int64_t groups,
+                       int64_t keep, const Tensor& ids, const Tensor& weights) {
+  TORCH_CHECK(z.dim() == 2, "moe_route_grouped: z [T, E]");
+  const int T = (int)z.size(0), E = (int)z.size(1);
+  TORCH_CHECK(top >= 1 && top <= E, "moe_route_grouped: top");
+  TORCH_CHECK(groups == 0 || (groups <= 64 && E % groups == 0 && keep >= 1 && keep <= groups &&
+                              top <= keep * (E / groups)), "moe_route_grouped: groups");
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kInt && ids.is_contiguous() &&
+              ids.numel() == (int64_t)T * top, "moe_route_grouped: ids [T, top] int32");
+  rfqmix::launch_moe_route_grouped(f32p(z, "z"), f32p(corr, "correction", E), T, E, (int)top,
+                                   (int)groups, (int)keep, ids.data_ptr<int32_t>(),
+                                   const_cast<float*>(f32p(weights, "weights", (int64_t)T * top)),
+                                   stream());
+}
+
+void moe_pair_up(const Tensor& h, const Tensor& ids, const Tensor& w13, const Tensor& act) {
+  const bool f32 = act_f32(h, "moe_pair_up h");
+  TORCH_CHECK(h.dim() == 2 && h.stride(1) == 1 && w13.dim() == 3 && w13.is_contiguous() &&
+              w13.is_cuda() && w13.scalar_type() == h.scalar_type() && w13.size(2) == h.size(1) &&
+              w13.size(1) % 2 == 0, "moe_pair_up: h [T, d], w13 [E, 2F, d]");
+  const int T = (int)h.size(0), d = (int)h.size(1), E = (int)w13.size(0), F = (int)w13.size(1) / 2;
+  const int pairs = (int)ids.numel();
+  TORCH_CHECK(T > 0 ? pairs % T == 0 : pairs == 0, "moe_pair_up: ids [T, top]");
+  TORCH_CHECK(rows2d(act, pairs, F) && act.is_contiguous() && act.scalar_type() == h.scalar_type(),
+              "moe_pair_up: act [T top, F]");
+  TORCH_CHECK((int64_t)d * 4 <= 64 * 1024 && (F + 63) / 64 <= 65535, "moe_pair_up: sizes");
+  rfqmix::launch_moe_pair_up(f32, h.data_ptr(), h.stride(0), i32p(ids, "ids", pairs), w13.data_ptr(),
+                             act.data_ptr(), pairs, T > 0 ? pairs / T : 1, d, F, E, stream());
+}
+
+void moe_pair_down(const Tensor& act, const Tensor& ids, const Tensor& weights, const Tensor& w2,
+                   const OptT& base, const Tensor& out) {
+  const bool f32 = act_f32(act, "moe_pair_down act");
+  TORCH_CHECK(out.dim() == 2 && w2.dim() == 3 && w2.is_contiguous() && w2.is_cuda() &&
+              w2.scalar_type() == act.scalar_type() && w2.size(1) == out.size(1),
+              "moe_pair_down: w2 [E, d, F], out [T, d]");
+  const int T = (int)out.size(0), d = (int)out.size(1), E = (int)w2.size(0), F = (int)w2.size(2);
+  const int pairs = (int)ids.numel(), top = T > 0 ? pairs / T : 1;
+  TORCH_CHECK(pairs == T * top && rows2d(act, pairs, F) && act.is_contiguous(), "moe_pair_down: act [T top, F]");
+  TORCH_CHECK((int64_t)top * F * 4 <= 160 * 1024 - 256 && (d + 63) / 64 <= 65535, "moe_pair_down: sizes");
+  const void* bp = nullptr;
+  int64_t bs = 0;
+  if (base.has_value()) {
+    TORCH_CHECK(base->is_cuda() && rows2d(*base, T, d) && base->scalar_type() == act.scalar_type(),
+                "moe_pair_down: base [T, d]");
+    bp = base->data_ptr();
+    bs = base->stride(0);
+  }
+  rfqmix::launch_moe_pair_down(f32, act.data_ptr(), i32p(ids, "ids", pairs),
+                               f32p(weights, "weights", pairs), w2.data_ptr(), bp, bs,
+                               const_cast<float*>(f32p(out, "out")), T, top, d, F, E, stream());
+}
+
 }  // namespace
 
 TORCH_LIBRARY(rfq_mix, m) {
@@ -262,6 +447,17 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("attn_mix_mfma(Tensor qn, Tensor ts, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor slopes, Tensor? sink, int chunk, bool grouped) -> ()");
   m.def("glu_clamped(Tensor gate_up, float limit, float alpha, Tensor(a!) out) -> ()");
   m.def("mixq_mfma_ok", &mixq_mfma_ok);
+  m.def("embed_rows(Tensor ids, Tensor table, Tensor(a!) out) -> ()");
+  m.def("post_norm_add(Tensor y, Tensor(a!) residual, Tensor w, float mult, float eps, Tensor(b!)? copy) -> ()");
+  m.def("rms_norm_rows(Tensor x, Tensor w, float eps, float offset, Tensor(a!) out) -> ()");
+  m.def("latent_norm_append(Tensor x, Tensor w, float eps, Tensor slots, Tensor(a!) pool) -> ()");
+  m.def("silu_mul_any(Tensor gate_up, Tensor(a!) out) -> ()");
+  m.def("softcap(Tensor(a!) x, float cap) -> ()");
+  m.def("token_shift_mix(Tensor x, Tensor mu, Tensor(a!) prev, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor(b!) out) -> ()");
+  m.def("wkv_recurrence(Tensor r, Tensor k, Tensor v, Tensor zw, Tensor w0, Tensor u, Tensor gate, Tensor norm_w, float eps, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor(b!) out) -> ()");
+  m.def("moe_route_grouped(Tensor z, Tensor correction, int top, int groups, int keep, Tensor(a!) ids, Tensor(b!) weights) -> ()");
+  m.def("moe_pair_up(Tensor h, Tensor ids, Tensor w13, Tensor(a!) act) -> ()");
+  m.def("moe_pair_down(Tensor act, Tensor ids, Tensor weights, Tensor w2, Tensor? base, Tensor(a!) out) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(rfq_mix, CUDA, m) {
@@ -273,4 +469,15 @@ TORCH_LIBRARY_IMPL(rfq_mix, CUDA, m) {
   m.impl("attn_mixq_prefill", &attn_mixq_prefill);
   m.impl("attn_mix_mfma", &attn_mix_mfma);
   m.impl("glu_clamped", &glu_clamped);
+  m.impl("embed_rows", &embed_rows);
+  m.impl("post_norm_add", &post_norm_add);
+  m.impl("rms_norm_rows", &rms_norm_rows);
+  m.impl("latent_norm_append", &latent_norm_append);
+  m.impl("silu_mul_any", &silu_mul_any);
+  m.impl("softcap", &softcap);
+  m.impl("token_shift_mix", &token_shift_mix);
+  m.impl("wkv_recurrence", &wkv_recurrence);
+  m.impl("moe_route_grouped", &moe_route_grouped);
+  m.impl("moe_pair_up", &moe_pair_up);
+  m.impl("moe_pair_down", &moe_pair_down);
 }

@@ -149,3 +149,13 @@ def forward(cfg, full, tokens, layers_out=None):
     y = norm_around_zero(x, W["final.norm"], eps) @ W["head"].T
     cap = cfg["logit_softcap"]
     return cap * torch.tanh(y / cap)
+
+
+def greedy(cfg, full, prompt, n):
+    """n tokens, each the argmax of the logits after everything before it."""
+    t, out = list(prompt), []
+    for _ in range(n):
+        nxt = int(forward(cfg, full, t)[-1].argmax())
+        out.append(nxt)
+        t.append(nxt)
+    return out
