@@ -75,9 +75,11 @@ def parse():
                     help="fraction of free HBM for the paged KV pool (288 GB per MI355X)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--arch-sizes", default="", help="--arch-compare: size classes, comma separated")
+    ap.add_argument("--arch-models", default="",
+                    help="--arch-compare: which of the two models to run (default both), comma separated")
     ap.add_argument("--arch-compare", default="",
-                    help="livisun: instead of the RFQ workload, time prefill and decode of the "
-                         "layer-list model beside the Llama decoder at equal layer sizes "
+                    help="livisun | numalorn: instead of the RFQ workload, time prefill and decode "
+                         "of the layer-list model beside the closest decoder at equal layer sizes "
                          "(replisense_rfq_amd/benchmarks/arch_compare.py); one JSON line")
     ap.add_argument("--time-budget", type=float, default=0.0,
                     help="seconds; if > 0 the latency phase is skipped once this much wall "
@@ -364,8 +366,8 @@ def main():
     args = parse()
     t_start = time.perf_counter()
     if args.arch_compare:
-        if args.arch_compare != "livisun" or args.gpus != 1:
-            raise SystemExit("bench: --arch-compare livisun runs on one GPU")
+        if args.arch_compare not in ("livisun", "numalorn") or args.gpus != 1:
+            raise SystemExit("bench: --arch-compare livisun | numalorn runs on one GPU")
         from replisense_rfq_amd.benchmarks import arch_compare
 
         print(json.dumps({"metric": "arch_compare", "arch": args.arch_compare, "dtype": "bf16",

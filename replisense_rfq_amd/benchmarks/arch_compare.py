@@ -1,5 +1,7 @@
-"""Prefill and decode throughput of a layer-list model beside the Llama decoder at equal
-layer sizes (``bench.py --arch-compare livisun``).
+"""Prefill and decode throughput of a layer-list model beside the closest decoder of the
+framework at equal layer sizes: ``bench.py --arch-compare livisun`` (beside Llama) and
+``--arch-compare numalorn`` (beside the Mixtral-style sparse decoder: same width, head count,
+experts, choices per token and expert width).
 
 Both run through the same engine (scheduler, paged cache, hipGraph decode steps), with
 random weights, a few layers of a real model's shape and a small vocabulary, so the numbers
@@ -10,6 +12,7 @@ compare the layers' kernels:
 """
 from __future__ import annotations
 
+import sys
 import time
 
 import torch
@@ -22,6 +25,8 @@ from ..utils.config import EngineConfig
 # (name, hidden, q heads, kv heads, ff) with 128-wide heads (the Llama kernels' head size)
 SIZES = [("1b-class", 2048, 16, 4, 8192), ("8b-class", 4096, 32, 8, 14336),
          ("70b-class", 8192, 64, 8, 28672)]
+# (name, hidden, q heads, kv heads of the sparse decoder, experts, choices, expert ff)
+MOE_SIZES = [("moe-2k", 2048, 16, 4, 8, 2, 4096), ("moe-4k", 4096, 32, 8, 8, 2, 14336)]
 LAYERS, VOCAB, CHUNK = 4, 32000, 2048
 
 
@@ -34,12 +39,38 @@ def _configs(name, d, H, G, F):
     return llama, liv
 
 
+def _moe_configs(name, d, H, G, E, top, F):
+    """Sparse decoder and Numalorn at equal sizes: latent attention with 128-wide heads, a
+    512-wide cached latent and a 3d/8 query latent, alternating with wkv layers of 64-wide
+    heads; the same experts, in two groups of which the better one is kept; no shared expert
+    (the sparse decoder has none)."""
+    from ..models.config import numalorn_layers
+
+    sparse = ModelConfig(f"cmp-sparse-{name}", vocab_size=VOCAB, hidden=d, n_layers=LAYERS,
+                         n_heads=H, n_kv_heads=G, ffn=F, n_experts=E, moe_topk=top, bos_id=1,
+                         eos_ids=())
+    num = LayeredConfig(f"cmp-numalorn-{name}", architecture="Numalorn", vocab_size=VOCAB,
+                        hidden=d, canon_taps=0, residual_mult=0.5, logit_softcap=30.0,
+                        decay_rank=64,
+                        layers=numalorn_layers(LAYERS, H, 128, 128, 3 * d // 8, 512, d // 64, F, E,
+                                               top, 2, 1, 0))
+    return sparse, num
+
+
 def _engine(mcfg, args, batch):
-    from ..models.livisun import LivisunLM
+    from ..models import layered_model_class
     from ..models.llama import DecoderLM
 
     dev = torch.device("cuda", 0)
-    model = (LivisunLM if isinstance(mcfg, LayeredConfig) else DecoderLM)(mcfg, dev, seed=args.seed)
+    if isinstance(mcfg, LayeredConfig) and mcfg.architecture == "Numalorn":
+        from ..models.weights import init_numalorn_weights
+
+        w = init_numalorn_weights(mcfg, dev, torch.bfloat16, args.seed, keep_full=False)
+        model = layered_model_class(mcfg.architecture)(mcfg, dev, weights=w)
+    elif isinstance(mcfg, LayeredConfig):
+        model = layered_model_class(mcfg.architecture)(mcfg, dev, seed=args.seed)
+    else:
+        model = DecoderLM(mcfg, dev, seed=args.seed)
     cfg = EngineConfig(model=mcfg.name, max_num_seqs=batch, max_kv_blocks=batch * 80 + 64,
                        max_batched_tokens=args.prefill_chunk, max_model_len=2560,
                        use_graphs=not args.no_graphs, graph_buckets=(batch,), grammar=False,
@@ -75,23 +106,34 @@ def run(args) -> dict:
     out = {"layers": LAYERS, "vocab": VOCAB, "block": CHUNK, "prompt": [8, 2048],
            "decode": [64, 128], "sizes": {}}
     only = [x for x in getattr(args, "arch_sizes", "").split(",") if x]
-    for name, d, H, G, F in SIZES:
+    arch = getattr(args, "arch_compare", "livisun")
+    base = "llama" if arch == "livisun" else "sparse"
+    for size in (SIZES if arch == "livisun" else MOE_SIZES):
+        name = size[0]
         if only and name not in only:
             continue
         row = {}
-        for mcfg in _configs(name, d, H, G, F):
-            kind = "livisun" if isinstance(mcfg, LayeredConfig) else "llama"
+        models = [x for x in getattr(args, "arch_models", "").split(",") if x]
+        for mcfg in (_configs(*size) if arch == "livisun" else _moe_configs(*size)):
+            kind = arch if isinstance(mcfg, LayeredConfig) else base
+            if models and kind not in models:
+                continue
+            print(f"[arch-compare] {name}: {kind}", file=sys.stderr, flush=True)
             eng = _engine(mcfg, args, 64)
             pre = [torch.randint(2, VOCAB, (2048,), generator=g).tolist() for _ in range(8)]
             dec = [torch.randint(2, VOCAB, (512,), generator=g).tolist() for _ in range(64)]
+            print("[arch-compare]   engine up; warm-up", file=sys.stderr, flush=True)
             _measure(eng, pre[:2], 2)                              # warm-up
+            print("[arch-compare]   prefill", file=sys.stderr, flush=True)
             p_tps, _, _ = _measure(eng, pre, 1)
+            print("[arch-compare]   decode", file=sys.stderr, flush=True)
             _, d_tps, steps = _measure(eng, dec, 128)
             row[kind] = {"prefill_tok_s": round(p_tps), "decode_tok_s": round(d_tps),
                          "decode_steps": steps, "graph_steps": eng.runner.stats["graph_steps"]}
             del eng
             torch.cuda.empty_cache()
-        row["prefill_ratio"] = round(row["livisun"]["prefill_tok_s"] / row["llama"]["prefill_tok_s"], 3)
-        row["decode_ratio"] = round(row["livisun"]["decode_tok_s"] / row["llama"]["decode_tok_s"], 3)
+        if arch in row and base in row:
+            row["prefill_ratio"] = round(row[arch]["prefill_tok_s"] / row[base]["prefill_tok_s"], 3)
+            row["decode_ratio"] = round(row[arch]["decode_tok_s"] / row[base]["decode_tok_s"], 3)
         out["sizes"][name] = row
     return out

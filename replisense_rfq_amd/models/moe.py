@@ -80,8 +80,12 @@ class MoEBuffers:
 
 def moe_mlp(x: torch.Tensor, router_w: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
             topk: int, bufs: MoEBuffers | None, out: torch.Tensor | None = None,
-            expert_offset: int = 0) -> torch.Tensor:
+            expert_offset: int = 0, routing=None) -> torch.Tensor:
     """x [T, d] -> [T, d].  w13 [E, 2F, d] (gate|up), w2 [E, d, F], router_w [E_all, d].
+
+    ``routing``: a callable (weights [T, topk] fp32, ids [T, topk] int32) that fills both for
+    this step's rows in place of the softmax top-k router (models with a router of their own;
+    GPU only); the alignment, expert GEMMs and weighted combine are the same.
 
     Expert parallelism: when this rank holds experts [expert_offset, expert_offset +
     E) of E_all, pairs routed elsewhere are sent to a dummy expert segment that no
@@ -103,7 +107,10 @@ def moe_mlp(x: torch.Tensor, router_w: torch.Tensor, w13: torch.Tensor, w2: torc
     if T <= SKINNY_MAX_TOKENS:
         # decode / short-extend steps: router GEMV + top-k in one kernel, stream only
         # the routed experts' weights, gather rows on the fly, SwiGLU fused into w13
-        ops.moe_route(x, router_w, topk, True, w, ids)
+        if routing is not None:
+            routing(w, ids)
+        else:
+            ops.moe_route(x, router_w, topk, True, w, ids)
         if ep:
             _localize(ids, w, expert_offset, E - 1)
         cap = (n + E * (BLOCK_S - 1) + BLOCK_S - 1) // BLOCK_S * BLOCK_S
@@ -125,10 +132,12 @@ def moe_mlp(x: torch.Tensor, router_w: torch.Tensor, w13: torch.Tensor, w2: torc
         ops.moe_skinny(act, sorted_ids, topk, bufs.expert_offsets, w2, y, False, False, n)
         ops.moe_combine(y, bufs.inv_pos[:n], w, topk, out)
         return out
-    logits = x @ router_w.t()
     cap = (n + E * (BLOCK_M - 1) + BLOCK_M - 1) // BLOCK_M * BLOCK_M
     nb = cap // BLOCK_M
-    ops.moe_topk(logits, topk, True, w, ids)
+    if routing is not None:
+        routing(w, ids)
+    else:
+        ops.moe_topk(x @ router_w.t(), topk, True, w, ids)
     if ep:
         _localize(ids, w, expert_offset, E - 1)
     sorted_ids, eob = bufs.sorted_ids[:cap], bufs.expert_of_block[:nb]
@@ -186,3 +195,17 @@ def _localize(ids: torch.Tensor, w: torch.Tensor, e0: int, e_local: int) -> None
     ids.copy_(torch.where(mine, loc, torch.full_like(loc, e_local)))
     w.mul_(mine.to(w.dtype))
 
+
+
+def grouped_ok(w13: torch.Tensor, w2: torch.Tensor) -> bool:
+    """Whether the expert kernels of this module take a model's experts (bf16 on the GPU, at
+    most 64 experts, widths of the skinny and of the dense grouped kernels) and their library
+    is built: a model with other sizes runs its own general expert kernels instead."""
+    from ..ops import _native
+
+    E, F2, d = w13.shape
+    F = F2 // 2
+    return bool(w13.is_cuda and w13.dtype == torch.bfloat16 and E <= 64 and d % 256 == 0 and
+                F % 256 == 0 and F >= 512 and ops.moe_gemm_dense_ok(w13, True) and
+                ops.moe_gemm_dense_ok(w2, False) and _native.lib_path().exists() and
+                _native.available())

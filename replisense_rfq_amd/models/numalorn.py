@@ -31,6 +31,7 @@ import torch
 from .. import ops
 from ..parallel.tp import SINGLE, TPContext
 from .config import LayeredConfig
+from .moe import MoEBuffers, grouped_ok, moe_mlp
 from .weights import init_numalorn_weights
 
 
@@ -55,9 +56,14 @@ class NumalornLM:
         self.norms_folded = False
         if dtype == torch.float32:
             torch.backends.cuda.matmul.allow_tf32 = False
+        self._moe_bufs: dict = {}
         for ly, lw in zip(cfg.layers, self.w["layers"]):
             if ly.mixer.kind == "latent_attention":
                 lw["no_slope"] = torch.zeros(ly.mixer.heads, dtype=torch.float32, device=self.device)
+            # experts whose sizes the framework's grouped MFMA expert GEMMs take run there
+            # (the sparse decoder's alignment, GEMMs and combine, behind this model's router)
+            lw["grouped"] = bool(ly.mlp is not None and self.device.type == "cuda"
+                                 and dtype == torch.bfloat16 and grouped_ok(lw["w13"], lw["w2e"]))
 
     # engine hooks shared with the other decoders
     def fold_norms(self) -> bool:
@@ -76,7 +82,7 @@ class NumalornLM:
     def weight_bytes(self) -> int:
         tot = sum(v.numel() * v.element_size() for v in self.w.values() if isinstance(v, torch.Tensor))
         for lw in self.w["layers"]:
-            tot += sum(t.numel() * t.element_size() for t in lw.values())
+            tot += sum(t.numel() * t.element_size() for t in lw.values() if isinstance(t, torch.Tensor))
         return tot
 
     # ------------------------------------------------------------------ mixers
@@ -119,15 +125,30 @@ class NumalornLM:
                                torch.empty((T, HN), dtype=dt, device=x.device))
         return ops.matmul_nt(y, lw["o"])
 
+    def _moe_buffers(self, T: int, f, d: int) -> MoEBuffers:
+        cap = 1
+        while cap < T:
+            cap *= 2
+        key = (cap, f.top, f.experts, f.ff)
+        if key not in self._moe_bufs:
+            self._moe_bufs[key] = MoEBuffers.allocate(cap, f.top, f.experts, d, f.ff, self.device,
+                                                      self.dtype)
+        return self._moe_bufs[key]
+
     def _moe(self, f, lw, h):
         T, dev = h.shape[0], h.device
         z = ops.matmul_nt(h.float(), lw["router"])
-        ids = torch.empty((T, f.top), dtype=torch.int32, device=dev)
-        wts = torch.empty((T, f.top), dtype=torch.float32, device=dev)
-        ops.moe_route_grouped(z, lw["correction"], f.top, f.groups, f.keep, ids, wts)
         base = None
         if f.shared_ff:
             base = ops.matmul_nt(ops.silu_mul_any(ops.matmul_nt(h, lw["shared_gu"])), lw["shared_down"])
+        if lw["grouped"]:
+            y = moe_mlp(h, lw["router"], lw["w13"], lw["w2e"], f.top, self._moe_buffers(T, f, h.shape[1]),
+                        routing=lambda w, i: ops.moe_route_grouped(z, lw["correction"], f.top,
+                                                                   f.groups, f.keep, i, w))
+            return y if base is None else y.float().add_(base)
+        ids = torch.empty((T, f.top), dtype=torch.int32, device=dev)
+        wts = torch.empty((T, f.top), dtype=torch.float32, device=dev)
+        ops.moe_route_grouped(z, lw["correction"], f.top, f.groups, f.keep, ids, wts)
         return ops.moe_experts(h, ids, wts, lw["w13"], lw["w2e"], base,
                                torch.empty((T, h.shape[1]), dtype=torch.float32, device=dev))
 

@@ -408,8 +408,11 @@ def _numalorn_assemble(get, has, cfg, device, dtype) -> dict:
             HN = m.heads * m.dim
             lw["mu"] = torch.stack([vec(p + "mix.mu." + s, d) for s in "rkvgw"]).contiguous()
             lw["rkvg"] = torch.stack([mat(p + "mix." + s, HN, d) for s in "rkvg"]).contiguous().to(device)
-            rank = get(p + "mix.w1").shape[0]
-            lw["w1"] = mat(p + "mix.w1", rank, d).contiguous().to(device)
+            w1 = get(p + "mix.w1")
+            rank = w1.shape[0]                       # the decay's inner size is the tensor's
+            if tuple(w1.shape) != (rank, d):
+                raise ValueError(f"tensor {p}mix.w1: shape {tuple(w1.shape)}, expected (rank, {d})")
+            lw["w1"] = w1.to(dtype).contiguous().to(device)
             lw["w2"] = mat(p + "mix.w2", HN, rank).contiguous().to(device)
             lw["w0"] = vec(p + "mix.w0", HN)
             lw["u"] = vec(p + "mix.u", m.heads, m.dim)
@@ -433,15 +436,21 @@ def _numalorn_assemble(get, has, cfg, device, dtype) -> dict:
     return w
 
 
-def init_numalorn_weights(cfg, device, dtype=torch.bfloat16, seed: int = 0) -> dict:
+def init_numalorn_weights(cfg, device, dtype=torch.bfloat16, seed: int = 0,
+                          keep_full: bool = True) -> dict:
     """Seeded random Numalorn weights under the checkpoint's names (tests and benchmarks):
     projections scaled so that activations stay O(1); sinks, corrections, bonuses, decays and
-    zero-centred norm weights away from their neutral values so that each shows in the logits."""
+    zero-centred norm weights away from their neutral values so that each shows in the logits.
+    ``keep_full`` False (benchmark sizes): drawn on the device, the name -> tensor dict is not
+    kept."""
     d, full = cfg.hidden, {}
 
     def rnd(name, shape, std, mean=0.0):
-        t = _randn(shape, std, (seed, name), "cpu", torch.float32) + mean
-        full[name] = t.to(torch.bfloat16).float()
+        if keep_full:
+            t = _randn(shape, std, (seed, name), "cpu", torch.float32) + mean
+            full[name] = t.to(torch.bfloat16).float()
+        else:
+            full[name] = (_randn(shape, std, (seed, name), device, torch.float32) + mean).to(torch.bfloat16)
         return full[name]
 
     rnd("embed", (cfg.vocab_size, d), 1.0)
@@ -488,6 +497,8 @@ def init_numalorn_weights(cfg, device, dtype=torch.bfloat16, seed: int = 0) -> d
                 rnd(q + "shared.gate", (f.shared_ff, d), d ** -0.5)
                 rnd(q + "shared.up", (f.shared_ff, d), d ** -0.5)
                 rnd(q + "shared.down", (d, f.shared_ff), f.shared_ff ** -0.5)
+    if not keep_full:
+        return _numalorn_assemble(lambda k: full.pop(k), lambda k: k in full, cfg, device, dtype)
     return numalorn_from_full(full, cfg, device, dtype)
 
 

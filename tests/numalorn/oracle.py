@@ -34,6 +34,26 @@ def shift_mix(h, mu):
     return h + (prev - h) * mu
 
 
+def decay(z, w0):
+    """Per-channel decay in (0, 1) from the decay projection's output."""
+    return torch.exp(-torch.exp(z + w0))
+
+
+def wkv_scan(r, k, v, w, u, S=None):
+    """Token by token per head: o_t = (S + diag(u) k_t v_t^T)^T r_t, then
+    S <- diag(w_t) S + k_t v_t^T.  r, k, v, w: [T, H, N]; u: [H, N]; S: [H, N, N] (key channel,
+    value channel), zeros at the start.  Returns (o [T, H, N], S)."""
+    T, H, N = r.shape
+    S = torch.zeros(H, N, N, dtype=F) if S is None else S.clone()
+    out = torch.zeros(T, H, N, dtype=F)
+    for t in range(T):
+        for hd in range(H):
+            kv = torch.outer(k[t, hd], v[t, hd])
+            out[t, hd] = (S[hd] + u[hd][:, None] * kv).T @ r[t, hd]
+            S[hd] = w[t, hd][:, None] * S[hd] + kv
+    return out, S
+
+
 def wkv_mixer(h, get, m, eps):
     """RWKV-style time mixing with a data-dependent decay and a bonus for the current token."""
     T, d = h.shape
@@ -43,16 +63,8 @@ def wkv_mixer(h, get, m, eps):
     k = (xk @ get("k").T).view(T, H, N)
     v = (xv @ get("v").T).view(T, H, N)
     gate = silu(xg @ get("g").T)
-    z = torch.tanh(xw @ get("w1").T) @ get("w2").T + get("w0")
-    w = torch.exp(-torch.exp(z)).view(T, H, N)
-    u = get("u").view(H, N)
-    out = torch.zeros(T, H, N, dtype=F)
-    for hd in range(H):
-        S = torch.zeros(N, N, dtype=F)                        # [key channel, value channel]
-        for t in range(T):
-            kv = torch.outer(k[t, hd], v[t, hd])
-            out[t, hd] = (S + u[hd][:, None] * kv).T @ r[t, hd]
-            S = w[t, hd][:, None] * S + kv
+    w = decay(torch.tanh(xw @ get("w1").T) @ get("w2").T, get("w0")).view(T, H, N)
+    out, _ = wkv_scan(r, k, v, w, get("u").view(H, N))
     out = rms_unit(out, eps).reshape(T, H * N) * get("norm") * gate
     return out @ get("o").T
 
