@@ -160,7 +160,9 @@ class LayeredConfig:
 
     @property
     def is_moe(self) -> bool:
-        return False
+        """Some layer routes tokens to experts: like the sparse decoder, decode graphs then
+        cover only steps small enough for the per-expert skinny kernels."""
+        return any(ly.mlp is not None and ly.mlp.kind == "moe" for ly in self.layers)
 
     def params(self) -> int:
         d, n = self.hidden, 0

@@ -137,7 +137,7 @@ class NumalornLM:
 
     def _moe(self, f, lw, h):
         T, dev = h.shape[0], h.device
-        z = ops.matmul_nt(h.float(), lw["router"])
+        z = ops.matmul_nt(h, lw["router"], out_dtype=torch.float32)
         base = None
         if f.shared_ff:
             base = ops.matmul_nt(ops.silu_mul_any(ops.matmul_nt(h, lw["shared_gu"])), lw["shared_down"])

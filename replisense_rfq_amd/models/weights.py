@@ -422,7 +422,9 @@ def _numalorn_assemble(get, has, cfg, device, dtype) -> dict:
         if f is not None:
             q = p + "mlp."
             lw["norm2"] = vec(p + "norm2", d)
-            lw["router"] = vec(q + "router", f.experts, d)
+            # the router's product accumulates and leaves in fp32; its operands are the
+            # checkpoint's weights in the model's dtype (exact: they are stored in bf16)
+            lw["router"] = mat(q + "router", f.experts, d).contiguous().to(device)
             lw["correction"] = vec(q + "correction", f.experts)
             lw["w13"] = torch.stack([torch.cat([mat(f"{q}e{e}.gate", f.ff, d), mat(f"{q}e{e}.up", f.ff, d)], 0)
                                      for e in range(f.experts)]).contiguous().to(device)

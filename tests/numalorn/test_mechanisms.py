@@ -120,7 +120,7 @@ def test_token_shift_two_sequences_in_one_launch(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("H,N", [(2, 64), (3, 24), (1, 7), (2, 96)])
+@pytest.mark.parametrize("H,N", [(2, 64), (3, 24), (1, 7), (2, 96), (32, 64)])
 @pytest.mark.parametrize("cuts", [[40], [1] * 40, [2, 1, 33, 4], [17, 2, 2, 19]])
 def test_wkv_recurrence_in_portions(device, H, N, cuts):
     """The recurrence in portions through a state slot with stale contents equals the scan of
@@ -221,7 +221,8 @@ def absorbed(q, uk, scale):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("H,dim,vdim,R", [(3, 16, 8, 24), (1, 8, 24, 40), (4, 32, 32, 64)])
+@pytest.mark.parametrize("H,dim,vdim,R", [(3, 16, 8, 24), (1, 8, 24, 40), (4, 32, 32, 64),
+                                          (16, 128, 128, 512)])
 def test_latent_attention_decode_rows(device, H, dim, vdim, R):
     """Rows of the decode section (1 to a few queries per sequence) over pages in odd order,
     lengths at page borders: scores and values both come from the one cached latent."""
@@ -237,7 +238,7 @@ def test_latent_attention_decode_rows(device, H, dim, vdim, R):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("H,dim,vdim,R", [(3, 16, 8, 24), (2, 8, 24, 72)])
+@pytest.mark.parametrize("H,dim,vdim,R", [(3, 16, 8, 24), (2, 8, 24, 72), (8, 128, 128, 512)])
 def test_latent_attention_prefill_rows_and_far_key(device, H, dim, vdim, R):
     """Portions of prompts behind cached tokens; one key far back (in the first page, at a page
     border) is made to dominate the last query's softmax over hundreds of others."""
@@ -360,6 +361,37 @@ def test_expert_products_and_weighted_sum(device, d, F, E, top, shared):
         base = ops.matmul_nt(ops.silu_mul_any(gu), W["shared.down"].to(device))
     out = ops.moe_experts(hd, ids, wts, w13, w2, base, torch.empty(T, d, device=device))
     close(out, want, 1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("d,F,E,top,groups,keep,T", [(512, 512, 8, 2, 2, 1, 300), (512, 512, 8, 2, 2, 1, 40),
+                                                     (1024, 1024, 16, 4, 4, 2, 700), (2048, 4096, 8, 2, 2, 1, 24)])
+def test_grouped_expert_gemms_match_the_general_kernels(d, F, E, top, groups, keep, T):
+    """bf16 experts whose sizes the sparse decoder's grouped GEMMs take run there behind this
+    router (few rows: per-expert skinny kernels; many: expert-sorted 128-row blocks, also with
+    experts that get no row); both agree with the general per-pair kernels."""
+    from replisense_rfq_amd.models.moe import MoEBuffers, grouped_ok, moe_mlp
+
+    dev = "cuda"
+    g = torch.Generator().manual_seed(12)
+    h = torch.randn(T, d, generator=g).bfloat16().to(dev)
+    w13 = (torch.randn(E, 2 * F, d, generator=g) * d ** -0.5).bfloat16().to(dev)
+    w2 = (torch.randn(E, d, F, generator=g) * F ** -0.5).bfloat16().to(dev)
+    z = (torch.randn(T, E, generator=g) * 2).to(dev)
+    corr = torch.randn(E, generator=g).to(dev)
+    corr[E // 2:] -= 50.0                                # the upper half never gets a row
+    assert grouped_ok(w13, w2)
+    ids = torch.empty(T, top, dtype=torch.int32, device=dev)
+    wts = torch.empty(T, top, device=dev)
+    ops.moe_route_grouped(z, corr, top, groups, keep, ids, wts)
+    assert int(ids.max()) < E // 2
+    want = ops.moe_experts(h, ids, wts, w13, w2, None, torch.empty(T, d, device=dev))
+    bufs = MoEBuffers.allocate(1 << (T - 1).bit_length(), top, E, d, F, dev, torch.bfloat16)
+    got = moe_mlp(h, z.new_zeros(E, d), w13, w2, top, bufs,
+                  routing=lambda w, i: ops.moe_route_grouped(z, corr, top, groups, keep, i, w))
+    torch.cuda.synchronize()
+    err = (got.float() - want).abs().max() / want.abs().max()
+    assert float(err) < 0.03, float(err)
 
 
 @pytest.mark.parametrize("device", DEVICES)

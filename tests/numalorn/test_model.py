@@ -198,3 +198,92 @@ def test_checkpoint_folder_round_trip(device, tmp_path):
     assert type(eng.model).__name__ == "NumalornLM"
     t = tokens(20, cfg["vocab"], 5)
     check(run_schedule(eng, alone(t, [9, 2])), cfg, full, {"a": t})
+
+
+@pytest.mark.gpu
+def test_layer_sized_model_in_bf16_against_the_torch_ops():
+    """Layers of a served model's widths (512-wide cached latent, 128-wide heads, 64-wide
+    recurrent heads, experts on the grouped GEMMs), bf16 on the GPU: prompts in portions and
+    decoding, against the same weights run in fp32 through the torch ops on the CPU."""
+    from .common import latent, moe, wkv, config
+
+    cfg = config([latent(8, 128, 128, 384, 512, 128 ** -0.5, moe(512, 8, 2, 2, 1)),
+                  wkv(16, 64, moe(512, 8, 2, 2, 1, 256)),
+                  latent(8, 128, 128, 384, 512, 128 ** -0.5, None, kv_from=0)],
+                 vocab=1000, width=1024, mult=0.5, cap=30.0)
+    kw = dict(max_kv_blocks=40, max_model_len=640, max_batched_tokens=1024)
+    ref_eng, full = build(cfg, "cpu", **kw)
+    eng, _ = build(cfg, "cuda:0", dtype=torch.bfloat16, full=full, **kw)
+    assert all(lw["grouped"] for lw, ly in zip(eng.model.w["layers"], cfg["layers"]) if ly["mlp"])
+    a, b = tokens(420, cfg["vocab"], 90), tokens(130, cfg["vocab"], 91)
+    steps = [{"entries": [("a", a[:300], [299]), ("b", b[:100], [0, 99])], "end": []},
+             {"entries": [("a", a[300:400], [0, 99]), ("b", b[100:101], [0])], "end": []}]
+    steps += [{"entries": [("a", a[400 + i:401 + i], [0]), ("b", b[101 + i:102 + i], [0])], "end": []}
+              for i in range(20)]
+    want = run_schedule(ref_eng, steps)
+    got = run_schedule(eng, steps)
+    assert len(got) == len(want) == 46
+    e = []
+    for key, row in got.items():
+        d = row.double() - want[key].double()
+        d = d - d.mean()
+        e.append(float(d.pow(2).mean().sqrt() / want[key].double().std()))
+    e.sort()
+    assert e[len(e) // 2] < 0.05 and e[-3] < 0.15, e[-6:]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decode_graphs_replayed_between_eager_steps(dtype):
+    """Decode steps replay a captured hipGraph (token shift, recurrence, latent attention,
+    routing and experts inside it), prompts run eagerly in between: greedy generation of
+    several waves of requests picks the oracle's tokens each time (fp32), and the graph was
+    the path that ran."""
+    from replisense_rfq_amd.engine.sequence import SamplingParams
+
+    cfg = HEAD64
+    eng, full = build(cfg, "cuda:0", dtype=dtype, use_graphs=True, graph_buckets=(4,))
+    assert eng.runner.graphs
+    for wave in range(3):
+        prompts = [tokens(n, cfg["vocab"], 100 + 10 * wave + n) for n in (9, 35, 2)]
+        seqs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, grammar=False))
+        if dtype == torch.float32:
+            for p, s in zip(prompts, seqs):
+                assert s.output_ids == oracle.greedy(cfg, full, p, 10), wave
+    assert eng.runner.stats["graph_steps"] >= 24
+    assert eng.core.num_free_state_slots == 4
+
+
+@pytest.mark.gpu
+def test_wide_layers_few_tokens_with_graphs():
+    """A 2048-wide layer pair (16 heads of 128 over a 512-wide latent, 32 recurrent heads,
+    8 experts of width 4096 on the grouped GEMMs) with decode graphs: a prompt in one eager
+    step, then graph steps; finite logits that do not depend on the path (graph or eager)."""
+    from replisense_rfq_amd.engine.sequence import SamplingParams
+    from .common import latent, moe, wkv, config
+
+    cfg = config([latent(16, 128, 128, 768, 512, 128 ** -0.5, moe(4096, 8, 2, 2, 1)),
+                  wkv(32, 64, moe(4096, 8, 2, 2, 1))], vocab=2000, width=2048, mult=0.5, cap=30.0)
+    from replisense_rfq_amd.models.config import numalorn_from_json
+    from replisense_rfq_amd.models.numalorn import NumalornLM
+    from replisense_rfq_amd.models.weights import init_numalorn_weights
+    from replisense_rfq_amd.engine.engine import LLMEngine
+    from replisense_rfq_amd.utils.config import EngineConfig
+
+    mcfg = numalorn_from_json(cfg, name="test-numalorn-wide")
+    outs = []
+    for graphs in (True, False):
+        w = init_numalorn_weights(mcfg, "cuda:0", torch.bfloat16, 0, keep_full=False)
+        model = NumalornLM(mcfg, "cuda:0", weights=w)
+        eng = LLMEngine(EngineConfig(model="x", device="cuda:0", max_num_seqs=4, max_kv_blocks=64,
+                                     max_batched_tokens=2048, max_model_len=512, use_graphs=graphs,
+                                     graph_buckets=(4,), grammar=False, prefix_cache=False,
+                                     warm_prefix=False, tune_gemm=False, jump_forward=False), model=model)
+        prompts = [tokens(n, cfg["vocab"], 200 + n) for n in (300, 70, 200)]
+        seqs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, grammar=False))
+        outs.append([s.output_ids for s in seqs])
+        assert bool(eng.runner.graphs) == graphs
+        del eng, model, w
+        torch.cuda.empty_cache()
+    same = sum(a == b for x, y in zip(*outs) for a, b in zip(x, y))
+    assert same >= 20, outs            # 24 tokens; a rounding tie may move a late one
