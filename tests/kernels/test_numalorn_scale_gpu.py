@@ -1,0 +1,153 @@
+"""Numalorn's kernels at the sizes of a served model's step (thousands of rows, 4096-wide
+layers, 32 attention and 64 recurrent heads) against the torch implementations of the same
+ops on the CPU."""
+import pytest
+import torch
+
+from replisense_rfq_amd import ops
+from replisense_rfq_amd.ops import reference as ref
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def i32(x):
+    return torch.tensor(x, dtype=torch.int32, device=DEV)
+
+
+def runs(lens, slots):
+    rs, rb, rf, pos = [], [], [], []
+    for n, s in zip(lens, slots):
+        rs += [2 * s] * n
+        rb += list(range(n))
+        rf += list(range(n - 1, -1, -1))
+        pos += list(range(n))
+    return rs, rb, rf, pos
+
+
+def rel(a, b):
+    return float((a.float().cpu() - b.float()).abs().max() / b.float().abs().max())
+
+
+def test_row_kernels_4096_wide():
+    g = torch.Generator().manual_seed(0)
+    T, d = 4096, 4096
+    x, y, w = torch.randn(T, d, generator=g), torch.randn(T, d, generator=g).bfloat16(), torch.randn(d, generator=g) * 0.3
+    xd, cp = x.to(DEV), torch.empty(T, d, dtype=torch.bfloat16, device=DEV)
+    ops.post_norm_add(y.to(DEV), xd, w.to(DEV), 0.5, 1e-5, cp)
+    ref.post_norm_add(y, x, w, 0.5, 1e-5, None)
+    assert rel(xd, x) < 1e-5 and rel(cp, x.bfloat16()) < 1e-2
+    mu = torch.rand(5, d, generator=g)
+    rs, rb, rf, pos = runs([2048, 2048], [0, 63])
+    prev_c, out_c = torch.zeros(128, d), torch.empty(5, T, d, dtype=torch.bfloat16)
+    ref.token_shift_mix(x, mu, prev_c, i32(rs).cpu(), i32(rb).cpu(), i32(rf).cpu(), i32(pos).cpu(), out_c)
+    prev_d, out_d = torch.zeros(128, d, device=DEV), torch.empty(5, T, d, dtype=torch.bfloat16, device=DEV)
+    ops.token_shift_mix(xd, mu.to(DEV), prev_d, i32(rs), i32(rb), i32(rf), i32(pos), out_d)
+    assert rel(out_d, out_c) < 1e-2 and rel(prev_d, prev_c) < 1e-6
+    wide = torch.randn(T, 2048, generator=g).bfloat16()
+    nw = torch.randn(1536, generator=g)
+    o_d = ops.rms_norm_rows(wide.to(DEV)[:, :1536], nw.to(DEV), 1e-5, torch.empty(T, 1536, dtype=torch.bfloat16, device=DEV))
+    o_c = torch.empty(T, 1536, dtype=torch.bfloat16)
+    ref.rms_norm_rows(wide[:, :1536], nw, 1e-5, o_c)
+    assert rel(o_d, o_c) < 1e-2
+
+
+def test_recurrence_64_heads_2048_token_runs():
+    g = torch.Generator().manual_seed(1)
+    H, N, lens = 64, 64, [2048, 2048]
+    T = sum(lens)
+    r, k, v, gate, zw = ((torch.randn(T, H * N, generator=g) * 0.5).bfloat16() for _ in range(5))
+    w0, u, nw = torch.randn(H * N, generator=g) - 2, torch.randn(H, N, generator=g) * 0.3, torch.ones(H * N)
+    rs, rb, rf, pos = runs(lens, [5, 63])
+    st_c, out_c = torch.zeros(128, H, N, N), torch.empty(T, H * N, dtype=torch.bfloat16)
+    # the torch op walks token by token: compare the first 200 tokens of each run and the
+    # final states of a shorter copy
+    sel = list(range(200)) + list(range(2048, 2248))
+    rs2, rb2, rf2, pos2 = runs([200, 200], [5, 63])
+    ref.wkv_recurrence(r[sel], k[sel], v[sel], zw[sel], w0, u, gate[sel], nw, 1e-5, st_c,
+                       i32(rs2).cpu(), i32(rb2).cpu(), i32(rf2).cpu(), i32(pos2).cpu(), out_c[:400])
+    st_d = torch.zeros(128, H, N, N, device=DEV)
+    out_d = torch.empty(T, H * N, dtype=torch.bfloat16, device=DEV)
+    ops.wkv_recurrence(*(a.to(DEV) for a in (r, k, v, zw)), w0.to(DEV), u.to(DEV), gate.to(DEV), nw.to(DEV),
+                       1e-5, st_d, i32(rs), i32(rb), i32(rf), i32(pos), out_d)
+    torch.cuda.synchronize()
+    assert rel(out_d[sel], out_c[:400]) < 2e-2
+    assert bool(torch.isfinite(out_d.float()).all()) and bool(torch.isfinite(st_d).all())
+
+
+def test_head_batched_products_4096_rows():
+    g = torch.Generator().manual_seed(2)
+    T, H, dim, R, vd = 4096, 32, 128, 512, 128
+    q = (torch.randn(T, H * dim, generator=g)).bfloat16()
+    uk = (torch.randn(H, dim, R, generator=g) * dim ** -0.5).bfloat16()
+    got = ops.bmm_f32(q.to(DEV).view(T, H, dim).transpose(0, 1), uk.to(DEV))
+    want = torch.bmm(q.float().view(T, H, dim).transpose(0, 1), uk.float())
+    assert rel(got, want) < 1e-2
+    lat = torch.randn(T, H * R, generator=g).bfloat16()
+    uvt = (torch.randn(H, R, vd, generator=g) * R ** -0.5).bfloat16()
+    got = torch.bmm(lat.to(DEV).view(T, H, R).transpose(0, 1), uvt.to(DEV))
+    want = torch.bmm(lat.float().view(T, H, R).transpose(0, 1), uvt.float())
+    assert rel(got, want) < 2e-2
+
+
+@pytest.mark.parametrize("d,F,T", [(2048, 4096, 4096), (4096, 14336, 4096)])
+def test_grouped_experts_4096_rows(d, F, T):
+    from replisense_rfq_amd.models.moe import MoEBuffers, grouped_ok, moe_mlp
+
+    g = torch.Generator(device=DEV).manual_seed(3)
+    E, top = 8, 2
+    h = torch.randn(T, d, generator=g, device=DEV).bfloat16()
+    w13 = (torch.randn(E, 2 * F, d, generator=g, device=DEV) * d ** -0.5).bfloat16()
+    w2 = (torch.randn(E, d, F, generator=g, device=DEV) * F ** -0.5).bfloat16()
+    z = torch.randn(T, E, generator=g, device=DEV) * 2
+    corr = torch.randn(E, generator=g, device=DEV) * 0.3
+    assert grouped_ok(w13, w2)
+    bufs = MoEBuffers.allocate(T, top, E, d, F, DEV, torch.bfloat16)
+    got = moe_mlp(h, z.new_zeros(E, d), w13, w2, top, bufs,
+                  routing=lambda w, i: ops.moe_route_grouped(z, corr, top, 2, 1, i, w))
+    torch.cuda.synchronize()
+    ids, wts = bufs.ids[:T].long(), bufs.weights[:T]
+    rows = torch.arange(0, T, 97, device=DEV)                 # a sample of rows, in torch
+    want = torch.zeros(rows.numel(), d, device=DEV)
+    for n, t in enumerate(rows.tolist()):
+        for j in range(top):
+            e = int(ids[t, j])
+            gu = h[t].float() @ w13[e].float().t()
+            a = (torch.nn.functional.silu(gu[:F]) * gu[F:]).bfloat16().float()
+            want[n] += wts[t, j] * (a @ w2[e].float().t())
+    assert rel(got[rows], want.cpu()) < 3e-2
+
+
+def test_latent_attention_32_heads_2048_token_prompts():
+    g = torch.Generator().manual_seed(4)
+    H, R, lens, BS = 32, 512, [2048, 600], 32
+    nblk = sum((n + BS - 1) // BS for n in lens) + 1
+    pool = (torch.randn(nblk, 1, BS, R, generator=g) * 0.5).bfloat16()
+    T = sum(lens)
+    qa = torch.randn(T, H, R, generator=g) * R ** -0.5
+    sink = torch.randn(H, generator=g)
+    maxb = (max(lens) + BS - 1) // BS
+    tables, at = [], 0
+    for n in lens:
+        nb = (n + BS - 1) // BS
+        tables.append(list(range(at, at + nb)) + [nblk - 1] * (maxb - nb))
+        at += nb
+    starts = [0, lens[0]]
+    work = [(s, b) for s, n in enumerate(lens) for b in range((n + 31) // 32)]
+    out_d = torch.empty(T, H * R, dtype=torch.bfloat16, device=DEV)
+    pd = pool.to(DEV)
+    ops.attn_mixq_prefill(qa.to(DEV), pd, pd, i32(tables), i32(starts), i32(lens), i32(lens),
+                          i32([w[0] for w in work]), i32([w[1] for w in work]), out_d,
+                          torch.zeros(H, device=DEV), sink.to(DEV), 0, 32)
+    torch.cuda.synchronize()
+    # the torch op on a sample of query rows: the second prompt whole, the end of the first
+    out_c = torch.empty(lens[1], H * R)
+    ref.attn_mixq_prefill(qa[lens[0]:], pool.float(), pool.float(), torch.tensor(tables[1:]), torch.tensor([0]),
+                          torch.tensor([lens[1]]), torch.tensor([lens[1]]), out_c, torch.zeros(H), sink, 0)
+    assert rel(out_d[lens[0]:], out_c) < 2e-2
+    tail = 64
+    out_t = torch.empty(tail, H * R)
+    ref.attn_mixq_prefill(qa[lens[0] - tail:lens[0]], pool.float(), pool.float(), torch.tensor(tables[:1]),
+                          torch.tensor([0]), torch.tensor([tail]), torch.tensor([lens[0]]), out_t,
+                          torch.zeros(H), sink, 0)
+    assert rel(out_d[lens[0] - tail:lens[0]], out_t) < 2e-2
