@@ -47,6 +47,11 @@ void launch_token_shift_mix(bool, const float*, const float*, float*, const int3
                             const int32_t*, const int32_t*, const int32_t*, void*, int, int, int,
                             int, hipStream_t);
 bool wkv_ok(int);
+bool latent_mfma_ok(int, int);
+bool launch_attn_latent_mfma(const void*, int64_t, int64_t, const void*, const int32_t*, int,
+                             const int32_t*, const int32_t*, const int32_t*, const int32_t*,
+                             const int32_t*, int, void*, int64_t, const float*, float, int, int, int,
+                             hipStream_t);
 void launch_wkv_recurrence(bool, const void*, const void*, const void*, const void*, const void*,
                            int64_t, int64_t, int64_t, int64_t, int64_t, const float*, const float*,
                            const float*, float, float*, const int32_t*, const int32_t*,
@@ -382,6 +387,38 @@ void wkv_recurrence(const Tensor& r, const Tensor& k, const Tensor& v, const Ten
       i32p(pos, "positions", T), out.data_ptr(), T, H, N, (int)state.size(0) / 2, stream());
 }
 
+// Latent attention on MFMA tiles: q [T, H, R] bf16 (the queries carried into the latent space;
+// any row and head strides that are multiples of 8), pool [blocks, 1, 32, R] bf16 = keys and
+// values, out [T, H R] bf16.
+void attn_latent_mfma(const Tensor& q, const Tensor& pool, const Tensor& bt, const Tensor& q_start,
+                      const Tensor& q_len, const Tensor& kv_len, const Tensor& work_seq,
+                      const Tensor& work_qblk, const Tensor& out, const OptT& sink, double scale) {
+  TORCH_CHECK(q.is_cuda() && q.scalar_type() == at::kBFloat16 && q.dim() == 3 && q.stride(2) == 1,
+              "attn_latent_mfma: q [T, H, R] bfloat16");
+  const int T = (int)q.size(0), H = (int)q.size(1), R = (int)q.size(2);
+  TORCH_CHECK(q.stride(0) % 8 == 0 && q.stride(1) % 8 == 0 &&
+              reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0, "attn_latent_mfma: q alignment");
+  TORCH_CHECK(pool.is_cuda() && pool.scalar_type() == at::kBFloat16 && pool.dim() == 4 &&
+              pool.is_contiguous() && pool.size(1) == 1 && pool.size(3) == R,
+              "attn_latent_mfma: pool [blocks, 1, BS, R] bfloat16");
+  const int BS = (int)pool.size(2), NB = (int)q_len.numel(), W = (int)work_seq.numel();
+  TORCH_CHECK(rfqmix::latent_mfma_ok(R, BS), "attn_latent_mfma: sizes outside the tiles");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == at::kBFloat16 && out.dim() == 2 &&
+              out.size(0) == T && out.size(1) == (int64_t)H * R && out.stride(1) == 1 &&
+              out.stride(0) % 4 == 0 && reinterpret_cast<uintptr_t>(out.data_ptr()) % 8 == 0,
+              "attn_latent_mfma: out [T, H R] bfloat16");
+  TORCH_CHECK(bt.dim() == 2 && bt.size(0) == NB, "attn_latent_mfma: block_tables [NB, maxb]");
+  TORCH_CHECK(work_qblk.numel() >= W, "attn_latent_mfma: work lists");
+  const bool ok = rfqmix::launch_attn_latent_mfma(
+      q.data_ptr(), q.stride(0), q.stride(1), pool.data_ptr(), i32p(bt, "block_tables", 0),
+      (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
+      i32p(kv_len, "kv_len", NB), i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W), W,
+      out.data_ptr(), out.stride(0), optf(sink, "sink", H), (float)scale, H, R, BS, stream());
+  TORCH_CHECK(ok, "attn_latent_mfma: no tile for these sizes");
+}
+
+bool latent_mfma_ok(int64_t R, int64_t BS) { return rfqmix::latent_mfma_ok((int)R, (int)BS); }
+
 void moe_route_grouped(const Tensor& z, const Tensor& corr, int64_t top, int64_t groups,
                        int64_t keep, const Tensor& ids, const Tensor& weights) {
   TORCH_CHECK(z.dim() == 2, "moe_route_grouped: z [T, E]");
@@ -447,6 +484,8 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("attn_mix_mfma(Tensor qn, Tensor ts, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor slopes, Tensor? sink, int chunk, bool grouped) -> ()");
   m.def("glu_clamped(Tensor gate_up, float limit, float alpha, Tensor(a!) out) -> ()");
   m.def("mixq_mfma_ok", &mixq_mfma_ok);
+  m.def("latent_mfma_ok", &latent_mfma_ok);
+  m.def("attn_latent_mfma(Tensor q, Tensor pool, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor? sink, float scale) -> ()");
   m.def("embed_rows(Tensor ids, Tensor table, Tensor(a!) out) -> ()");
   m.def("post_norm_add(Tensor y, Tensor(a!) residual, Tensor w, float mult, float eps, Tensor(b!)? copy) -> ()");
   m.def("rms_norm_rows(Tensor x, Tensor w, float eps, float offset, Tensor(a!) out) -> ()");
@@ -469,6 +508,7 @@ TORCH_LIBRARY_IMPL(rfq_mix, CUDA, m) {
   m.impl("attn_mixq_prefill", &attn_mixq_prefill);
   m.impl("attn_mix_mfma", &attn_mix_mfma);
   m.impl("glu_clamped", &glu_clamped);
+  m.impl("attn_latent_mfma", &attn_latent_mfma);
   m.impl("embed_rows", &embed_rows);
   m.impl("post_norm_add", &post_norm_add);
   m.impl("rms_norm_rows", &rms_norm_rows);

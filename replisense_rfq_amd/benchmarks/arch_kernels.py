@@ -1,0 +1,158 @@
+"""Per-kernel times of Numalorn's layer kernels at the sizes of a served model's steps
+(``bench.py --arch-compare numalorn``): a prefill step of 4,096 rows and a decode step of 64
+rows on 4096-wide layers (32 heads over a 512-wide cached latent, 64 recurrent heads of 64,
+8 experts of width 14,336 with 2 per token), bf16, random inputs.
+
+Each entry: time (HIP events, median of the repeats), the bytes the kernel has to move and
+the arithmetic it has to do, and ``distance`` = time / max(bytes / 8 TB/s, flops / 2.5 PFLOP/s).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+
+HBM, MFMA = 8e12, 2.5e15
+DEV = "cuda"
+
+
+def _time(fn, reps=20, warm=5):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        ts.append(a.elapsed_time(b) * 1e-3)
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def _entry(t, nbytes, flops):
+    floor = max(nbytes / HBM, flops / MFMA)
+    return {"us": round(t * 1e6, 1), "mbytes": round(nbytes / 1e6, 1), "gflop": round(flops / 1e9, 2),
+            "floor_us": round(floor * 1e6, 2), "distance": round(t / floor, 1)}
+
+
+def _i32(x):
+    return torch.tensor(x, dtype=torch.int32, device=DEV)
+
+
+def _runs(lens, slots, first=0):
+    """Per-row state arrays of runs of the given lengths that start at position ``first``."""
+    rs, rb, rf, pos = [], [], [], []
+    for n, s in zip(lens, slots):
+        rs += [2 * s] * n
+        rb += list(range(n))
+        rf += list(range(n - 1, -1, -1))
+        pos += list(range(first, first + n))
+    return _i32(rs), _i32(rb), _i32(rf), _i32(pos)
+
+
+def _rows(T, d, lens, slots, out, first=0):
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = torch.randn(T, d, generator=g, device=DEV)
+    y = torch.randn(T, d, generator=g, device=DEV).bfloat16()
+    w = torch.randn(d, generator=g, device=DEV) * 0.3
+    cp = torch.empty(T, d, dtype=torch.bfloat16, device=DEV)
+    out["post_norm_add"] = _entry(_time(lambda: ops.post_norm_add(y, x, w, 0.5, 1e-5, cp)), T * d * 12, 0)
+    mu = torch.rand(5, d, generator=g, device=DEV)
+    prev = torch.zeros(128, d, device=DEV)
+    rows = _runs(lens, slots, first)
+    mixes = torch.empty(5, T, d, dtype=torch.bfloat16, device=DEV)
+    out["token_shift_mix"] = _entry(_time(lambda: ops.token_shift_mix(x, mu, prev, *rows, mixes)), T * d * 14, 0)
+    return rows
+
+
+def _wkv(T, H, N, rows, out, decode):
+    g = torch.Generator(device=DEV).manual_seed(1)
+    r, k, v, gate, zw = ((torch.randn(T, H * N, generator=g, device=DEV) * 0.5).bfloat16() for _ in range(5))
+    w0 = torch.randn(H * N, generator=g, device=DEV) - 2
+    u = torch.randn(H, N, generator=g, device=DEV) * 0.3
+    nw = torch.ones(H * N, device=DEV)
+    st = torch.zeros(128, H, N, N, device=DEV)
+    y = torch.empty(T, H * N, dtype=torch.bfloat16, device=DEV)
+    t = _time(lambda: ops.wkv_recurrence(r, k, v, zw, w0, u, gate, nw, 1e-5, st, *rows, y))
+    seqs = int((rows[1] == 0).sum())
+    nbytes = T * H * N * 12 + (2 if decode else 1) * seqs * H * N * N * 4
+    out["wkv_recurrence"] = _entry(t, nbytes, 6.0 * T * H * N * N)
+
+
+def _attention(H, R, lens, q_lens, out, name):
+    g = torch.Generator(device=DEV).manual_seed(2)
+    BS = 32
+    nblk = sum((n + BS - 1) // BS for n in lens) + 1
+    pool = (torch.randn(nblk, 1, BS, R, generator=g, device=DEV) * 0.5).bfloat16()
+    T = sum(q_lens)
+    qa = torch.randn(T, H, R, generator=g, device=DEV) * R ** -0.5
+    sink = torch.randn(H, generator=g, device=DEV)
+    maxb = (max(lens) + BS - 1) // BS
+    tables, at = [], 0
+    for n in lens:
+        nb = (n + BS - 1) // BS
+        tables.append(list(range(at, at + nb)) + [nblk - 1] * (maxb - nb))
+        at += nb
+    starts = [sum(q_lens[:i]) for i in range(len(lens))]
+    lat = torch.empty(T, H * R, dtype=torch.bfloat16, device=DEV)
+    zero = torch.zeros(H, device=DEV)
+    bt, qs, ql, kl = _i32(tables), _i32(starts), _i32(q_lens), _i32(lens)
+    pairs = sum(q * (n - q) + q * (q + 1) // 2 for n, q in zip(lens, q_lens))
+    flops = 4.0 * R * H * pairs
+    if name == "decode":
+        t = _time(lambda: ops.attn_talk_decode(qa, pool, pool, bt, qs, ql, kl, lat, zero, None, sink, 1.0, 0))
+        out["attn_talk_decode (latent)"] = _entry(t, sum(lens) * R * 2 + T * H * R * 6, flops)
+    else:
+        work = [(s, b) for s, n in enumerate(q_lens) for b in range((n + 31) // 32)]
+        ws, wq = _i32([w[0] for w in work]), _i32([w[1] for w in work])
+        t = _time(lambda: ops.attn_mixq_prefill(qa, pool, pool, bt, qs, ql, kl, ws, wq, lat, zero, sink, 0, 32),
+                  reps=5, warm=1)
+        out["attn_mixq_prefill (latent)"] = _entry(t, sum(lens) * R * 2 + T * H * R * 6, flops)
+
+
+def _experts(T, d, F, E, top, out):
+    from ..models.moe import MoEBuffers, grouped_ok, moe_mlp
+
+    g = torch.Generator(device=DEV).manual_seed(3)
+    h = torch.randn(T, d, generator=g, device=DEV).bfloat16()
+    w13 = (torch.randn(E, 2 * F, d, generator=g, device=DEV) * d ** -0.5).bfloat16()
+    w2 = (torch.randn(E, d, F, generator=g, device=DEV) * F ** -0.5).bfloat16()
+    z = torch.randn(T, E, generator=g, device=DEV) * 2
+    corr = torch.randn(E, generator=g, device=DEV) * 0.3
+    ids = torch.empty(T, top, dtype=torch.int32, device=DEV)
+    wts = torch.empty(T, top, device=DEV)
+    out["moe_route_grouped"] = _entry(_time(lambda: ops.moe_route_grouped(z, corr, top, 2, 1, ids, wts)),
+                                      T * (E * 4 + top * 8), 0)
+    if not grouped_ok(w13, w2):
+        return
+    bufs = MoEBuffers.allocate(T, top, E, d, F, DEV, torch.bfloat16)
+    dummy = z.new_zeros(E, d)
+    t = _time(lambda: moe_mlp(h, dummy, w13, w2, top, bufs,
+                              routing=lambda w, i: ops.moe_route_grouped(z, corr, top, 2, 1, i, w)),
+              reps=10, warm=2)
+    used = min(E, T * top)
+    out["experts (route + grouped GEMMs + combine)"] = _entry(
+        t, used * 3 * d * F * 2 + T * d * 4, 6.0 * T * top * d * F)
+
+
+def run(args) -> dict:
+    torch.manual_seed(0)
+    d, H, R, WH, N, E, top, F = 4096, 32, 512, 64, 64, 8, 2, 14336
+    res = {"width": d, "heads": H, "latent": R, "recurrent_heads": [WH, N], "experts": [E, top, F]}
+    pre = {}
+    rows = _rows(4096, d, [2048, 2048], [0, 63], pre)
+    _wkv(4096, WH, N, rows, pre, False)
+    _attention(H, R, [2048, 600], [2048, 600], pre, "prefill")
+    _experts(4096, d, F, E, top, pre)
+    res["prefill_step_4096_rows"] = pre
+    dec = {}
+    rows = _rows(64, d, [1] * 64, list(range(64)), dec, first=600)
+    _wkv(64, WH, N, rows, dec, True)
+    # decode attention at 16 heads: its key tile still fits the LDS four times over
+    _attention(16, R, [600] * 64, [1] * 64, dec, "decode")
+    _experts(64, d, F, E, top, dec)
+    res["decode_step_64_rows"] = dec
+    return res

@@ -49,19 +49,24 @@ class NumalornLM:
         self.w = weights if weights is not None else init_numalorn_weights(cfg, self.device, dtype, seed)
         self.vocab_start = 0
         self.vocab_local = self.w["lm_head"].shape[0]
-        att = [ly.mixer.heads for ly in cfg.layers if ly.mixer.kind == "latent_attention"]
-        self.hq = max(att) if att else 1
-        self.hkv = 1
+        # what the scheduler sizes the decode kernels' work lists by (column tiles of hq / hkv
+        # heads per row): this model's kernels take none, one entry per row is the smallest
+        self.hq = self.hkv = 1
         self.kv_k = self.kv_v = self.layer_state = None
         self.norms_folded = False
         if dtype == torch.float32:
             torch.backends.cuda.matmul.allow_tf32 = False
         self._moe_bufs: dict = {}
+        self._seq_ids = None            # work list of the decode section: sequence j, block 0
         for ly, lw in zip(cfg.layers, self.w["layers"]):
             if ly.mixer.kind == "latent_attention":
                 lw["no_slope"] = torch.zeros(ly.mixer.heads, dtype=torch.float32, device=self.device)
             # experts whose sizes the framework's grouped MFMA expert GEMMs take run there
             # (the sparse decoder's alignment, GEMMs and combine, behind this model's router)
+            # bf16 on the GPU with a latent width the MFMA tiles cover: both sections run the
+            # MFMA latent attention; otherwise the general FMA kernels
+            lw["mfma"] = bool(ly.mixer.kind == "latent_attention" and self.device.type == "cuda"
+                              and dtype == torch.bfloat16 and ops.latent_mfma_ok(ly.mixer.kv_rank))
             lw["grouped"] = bool(ly.mlp is not None and self.device.type == "cuda"
                                  and dtype == torch.bfloat16 and grouped_ok(lw["w13"], lw["w2e"]))
 
@@ -78,6 +83,15 @@ class NumalornLM:
         [2*slots, d] fp32 for the wkv layers."""
         assert len(k_pools) == self.cfg.n_layers
         self.kv_k, self.kv_v, self.layer_state = k_pools, v_pools, layer_state
+
+    def _decode_work(self, n: int):
+        """(sequence index, query block 0) per decode-section sequence; views of two tensors
+        that only grow (never inside a graph capture: the warm-up run sizes them)."""
+        if self._seq_ids is None or self._seq_ids[0].numel() < n:
+            size = max(1024, 2 * n)
+            self._seq_ids = (torch.arange(size, dtype=torch.int32, device=self.device),
+                             torch.zeros(size, dtype=torch.int32, device=self.device))
+        return self._seq_ids[0][:n], self._seq_ids[1][:n]
 
     def weight_bytes(self) -> int:
         tot = sum(v.numel() * v.element_size() for v in self.w.values() if isinstance(v, torch.Tensor))
@@ -96,10 +110,24 @@ class NumalornLM:
         if mx.kv_from < 0:
             ops.latent_norm_append(dn[:, mx.q_rank:], lw["dkv_norm"], eps, m.slot_mapping[:T], pool)
         q = ops.matmul_nt(cq, lw["uq"]).view(T, H, mx.dim)
+        lat = torch.empty((T, H * R), dtype=dt, device=h.device)
+        if lw["mfma"]:
+            # queries carried into the latent space, [H, T, R] as the batched product leaves
+            # them; the kernel reads them through strides and scales the scores in fp32
+            qa = torch.bmm(q.transpose(0, 1), lw["uk"]).transpose(0, 1)
+            if D > 0:
+                ids, zeros = self._decode_work(m.dec_q_len.shape[0])
+                ops.attn_latent_mfma(qa[:D], pool, m.dec_block_tables, m.dec_q_start, m.dec_q_len,
+                                     m.dec_kv_len, ids, zeros, lat[:D], lw["sink"], mx.scale)
+            if T > D:
+                ops.attn_latent_mfma(qa[D:], pool, m.pf_block_tables, m.pf_q_start, m.pf_q_len,
+                                     m.pf_kv_len, m.work_seq, m.work_qblk, lat[D:T], lw["sink"],
+                                     mx.scale)
+            ov = torch.bmm(lat.view(T, H, R).transpose(0, 1), lw["uv_t"])
+            return ops.matmul_nt(ov.transpose(0, 1).reshape(T, H * mx.vdim), lw["o"])
         # absorbed queries, fp32 (they are score operands): [H, T, R] -> [T, H, R], scaled
         qa = torch.empty((T, H, R), dtype=torch.float32, device=h.device)
         torch.mul(ops.bmm_f32(q.transpose(0, 1), lw["uk"]).transpose(0, 1), mx.scale, out=qa)
-        lat = torch.empty((T, H * R), dtype=dt, device=h.device)
         if D > 0:
             ops.attn_talk_decode(qa[:D], pool, pool, m.dec_block_tables, m.dec_q_start,
                                  m.dec_q_len, m.dec_kv_len, lat[:D], lw["no_slope"], None,

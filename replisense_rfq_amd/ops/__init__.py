@@ -1160,6 +1160,28 @@ def bmm_f32(a, b):
     return torch.bmm(a.float(), b.float())
 
 
+LATENT_MFMA = os.environ.get("RFQ_LATENT_MFMA", "1") != "0"     # bf16: MFMA tiles where sizes fit
+
+
+def latent_mfma_ok(R: int, block: int = 32) -> bool:
+    """Whether the MFMA latent attention covers this latent width (bf16 pools, GPU)."""
+    return bool(LATENT_MFMA and _native.mix_ops().latent_mfma_ok(R, block))
+
+
+def attn_latent_mfma(q, pool, block_tables, q_start, q_len, kv_len, work_seq, work_qblk, out, sink,
+                     scale: float):
+    """Causal multi-query attention over the cached latents, which are keys and values at
+    once: q [T, H, R] bf16 holds the queries carried into the latent space (unscaled; any row
+    and head strides), out [T, H R] the weighted latents.  Work items (sequence, block of 32
+    queries) as for attn_mixq_prefill; the softmax's denominator holds exp(sink_h)."""
+    if _gpu(q):
+        _native.mix_ops().attn_latent_mfma(q, pool, block_tables, q_start, q_len, kv_len, work_seq,
+                                           work_qblk, out, sink, float(scale))
+    else:
+        ref.attn_mixq_prefill(q.float() * scale, pool, pool, block_tables, q_start, q_len, kv_len,
+                              out, torch.zeros(q.shape[1]), sink, 0)
+
+
 def embed_rows(ids, table, out=None):
     out = torch.empty((ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device) \
         if out is None else out

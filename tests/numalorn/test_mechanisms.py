@@ -258,6 +258,60 @@ def test_latent_attention_prefill_rows_and_far_key(device, H, dim, vdim, R):
         close(got, want, 1e-4)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,R", [(3, 64), (8, 128), (5, 256), (16, 512), (32, 512)])
+def test_latent_attention_on_matrix_cores(H, R):
+    """bf16 pools with a latent width of the MFMA tiles: decode rows and portions of prompts
+    behind cached tokens, pages in odd order, lengths at page borders, one far key that
+    dominates a late query, any head count; against the softmax over the same rounded rows."""
+    dev = "cuda"
+    g = torch.Generator().manual_seed(13)
+    lens, q_lens = [1, 32, 33, 97, 300, 70, 5, 64], [1, 1, 2, 3, 45, 70, 5, 33]
+    nblk = sum((n + BS - 1) // BS for n in lens) + 2
+    order = torch.randperm(nblk - 1, generator=g).tolist()
+    pool = (torch.randn(nblk, 1, BS, R, generator=g) * 9).bfloat16()              # stale everywhere
+    sink = torch.randn(H, generator=g)
+    scale = 0.41 * R ** -0.5
+    maxb = max((n + BS - 1) // BS for n in lens)
+    tables, qs, want = [], [], []
+    for n, ql in zip(lens, q_lens):
+        c = torch.randn(n, R, generator=g).bfloat16()
+        q = (torch.randn(ql, H, R, generator=g) * 3).bfloat16()
+        if n > 200:                                    # key 31 answers the last query of head H-1
+            c[31] = 0
+            c[31, 7] = 8.0
+            q[-1, H - 1] = 0
+            q[-1, H - 1, 7] = 40.0 / (8.0 * scale)
+        blocks = [order.pop() for _ in range((n + BS - 1) // BS)]
+        for p in range(n):
+            pool[blocks[p // BS], 0, p % BS] = c[p]
+        tables.append(blocks + [nblk - 1] * (maxb - len(blocks)))
+        qs.append(q)
+        cd, o = c.double(), torch.zeros(ql, H, R, dtype=D64)
+        for a in range(ql):
+            i = n - ql + a
+            sc = torch.einsum("hr,nr->hn", q[a].double(), cd[:i + 1]) * scale
+            mx = torch.maximum(sc.max(-1).values, sink.double())
+            e = torch.exp(sc - mx[:, None])
+            o[a] = (e @ cd[:i + 1]) / (e.sum(-1) + torch.exp(sink.double() - mx))[:, None]
+        want.append(o.reshape(ql, H * R))
+    want = torch.cat(want)
+    T = sum(q_lens)
+    # queries as the batched product leaves them: [H, T, R], read through strides
+    qh = torch.cat(qs).transpose(0, 1).contiguous().to(dev)
+    starts = [sum(q_lens[:i]) for i in range(len(lens))]
+    work = [(s_, b) for s_, ql in enumerate(q_lens) for b in range((ql + 31) // 32)]
+    out = torch.full((T, H * R), float("nan"), dtype=torch.bfloat16, device=dev)
+    ops.attn_latent_mfma(qh.transpose(0, 1), pool.to(dev), i32(tables, dev), i32(starts, dev),
+                         i32(q_lens, dev), i32(lens, dev), i32([w[0] for w in work], dev),
+                         i32([w[1] for w in work], dev), out, sink.to(dev), scale)
+    torch.cuda.synchronize()
+    err = (out.double().cpu() - want).abs().max() / want.abs().max()
+    assert float(err) < 1e-2, float(err)
+    far = want[sum(q_lens[:5]) - 1].view(H, R)[H - 1]
+    assert float(far[7]) > 7.5                         # the boosted key carries the row
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_sink_takes_weight_without_a_value(device):
     """One key with score 0 and a sink logit of ln 3: the output is a quarter of the value."""
