@@ -78,20 +78,34 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(
   float l_run = (sink != nullptr && cvalid) ? 1.f : 0.f;
   const bf16_t* ka = c_lds + c * RS + 8 * g4;          // this lane's A-fragment rows
 
+  // Page pipeline: the next page is loaded into registers while this one is multiplied out of
+  // LDS (one memory round trip per page, hidden behind the MFMAs).  Rows past the last key are
+  // zeroed: they may hold anything, and 0 * NaN would poison the weighted sum.
+  constexpr int NK = (kLatPg * (R / 8) + 255) / 256;
+  s16x8 creg[NK];
+  auto fetch = [&](int pg) {
+    const s16x8* cb = reinterpret_cast<const s16x8*>(pool + (int64_t)bt[pg] * kLatPg * R);
+#pragma unroll
+    for (int u = 0; u < NK; ++u) {
+      const int x = threadIdx.x + u * 256;
+      if (x < kLatPg * (R / 8))
+        creg[u] = pg * kLatPg + x / (R / 8) > plast ? (s16x8){0, 0, 0, 0, 0, 0, 0, 0} : cb[x];
+    }
+  };
   const int pg_last = plast / kLatPg;
+  fetch(0);
   for (int pg = 0; pg <= pg_last; ++pg) {
     const int kt = pg * kLatPg;
-    {
-      // straight copy of the page into LDS; rows past the last key are zeroed (they may hold
-      // anything, and 0 * NaN would poison the weighted sum)
-      const s16x8* cb = reinterpret_cast<const s16x8*>(pool + (int64_t)bt[pg] * kLatPg * R);
-      for (int x = threadIdx.x; x < kLatPg * (R / 8); x += 256) {
+#pragma unroll
+    for (int u = 0; u < NK; ++u) {
+      const int x = threadIdx.x + u * 256;
+      if (x < kLatPg * (R / 8)) {
         const int row = x / (R / 8), x8 = x - row * (R / 8);
-        const s16x8 v = kt + row > plast ? (s16x8){0, 0, 0, 0, 0, 0, 0, 0} : cb[x];
-        *reinterpret_cast<s16x8*>(c_lds + row * RS + 8 * x8) = v;
+        *reinterpret_cast<s16x8*>(c_lds + row * RS + 8 * x8) = creg[u];
       }
     }
     __syncthreads();                                   // tile visible
+    if (pg < pg_last) fetch(pg + 1);
     if (active) {
       constexpr int KF = EK < 8 ? EK : 8;
       f32x4 sc[2] = {(f32x4){0.f, 0.f, 0.f, 0.f}, (f32x4){0.f, 0.f, 0.f, 0.f}};

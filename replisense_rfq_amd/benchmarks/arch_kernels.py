@@ -82,7 +82,7 @@ def _wkv(T, H, N, rows, out, decode):
     out["wkv_recurrence"] = _entry(t, nbytes, 6.0 * T * H * N * N)
 
 
-def _attention(H, R, lens, q_lens, out, name):
+def _attention(H, R, lens, q_lens, out, name, mfma=False):
     g = torch.Generator(device=DEV).manual_seed(2)
     BS = 32
     nblk = sum((n + BS - 1) // BS for n in lens) + 1
@@ -102,15 +102,20 @@ def _attention(H, R, lens, q_lens, out, name):
     bt, qs, ql, kl = _i32(tables), _i32(starts), _i32(q_lens), _i32(lens)
     pairs = sum(q * (n - q) + q * (q + 1) // 2 for n, q in zip(lens, q_lens))
     flops = 4.0 * R * H * pairs
-    if name == "decode":
+    work = [(s, b) for s, n in enumerate(q_lens) for b in range((n + 31) // 32)]
+    ws, wq = _i32([w[0] for w in work]), _i32([w[1] for w in work])
+    if mfma:
+        qh = qa.bfloat16().transpose(0, 1).contiguous().transpose(0, 1)       # [H, T, R] in memory
+        t = _time(lambda: ops.attn_latent_mfma(qh, pool, bt, qs, ql, kl, ws, wq, lat, sink, 1.0),
+                  reps=10, warm=2)
+        out[f"attn_latent_mfma ({name})"] = _entry(t, sum(lens) * R * 2 + T * H * R * 4, flops)
+    elif name == "decode":
         t = _time(lambda: ops.attn_talk_decode(qa, pool, pool, bt, qs, ql, kl, lat, zero, None, sink, 1.0, 0))
-        out["attn_talk_decode (latent)"] = _entry(t, sum(lens) * R * 2 + T * H * R * 6, flops)
+        out["attn_talk_decode (latent, general FMA)"] = _entry(t, sum(lens) * R * 2 + T * H * R * 6, flops)
     else:
-        work = [(s, b) for s, n in enumerate(q_lens) for b in range((n + 31) // 32)]
-        ws, wq = _i32([w[0] for w in work]), _i32([w[1] for w in work])
         t = _time(lambda: ops.attn_mixq_prefill(qa, pool, pool, bt, qs, ql, kl, ws, wq, lat, zero, sink, 0, 32),
-                  reps=5, warm=1)
-        out["attn_mixq_prefill (latent)"] = _entry(t, sum(lens) * R * 2 + T * H * R * 6, flops)
+                  reps=3, warm=1)
+        out["attn_mixq_prefill (latent, general FMA)"] = _entry(t, sum(lens) * R * 2 + T * H * R * 6, flops)
 
 
 def _experts(T, d, F, E, top, out):
@@ -145,13 +150,15 @@ def run(args) -> dict:
     pre = {}
     rows = _rows(4096, d, [2048, 2048], [0, 63], pre)
     _wkv(4096, WH, N, rows, pre, False)
+    _attention(H, R, [2048, 600], [2048, 600], pre, "prefill", mfma=True)
     _attention(H, R, [2048, 600], [2048, 600], pre, "prefill")
     _experts(4096, d, F, E, top, pre)
     res["prefill_step_4096_rows"] = pre
     dec = {}
     rows = _rows(64, d, [1] * 64, list(range(64)), dec, first=600)
     _wkv(64, WH, N, rows, dec, True)
-    # decode attention at 16 heads: its key tile still fits the LDS four times over
+    _attention(H, R, [600] * 64, [1] * 64, dec, "decode", mfma=True)
+    # the general kernel at 16 heads: its key tile still fits the LDS four times over
     _attention(16, R, [600] * 64, [1] * 64, dec, "decode")
     _experts(64, d, F, E, top, dec)
     res["decode_step_64_rows"] = dec
