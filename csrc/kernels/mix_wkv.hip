@@ -61,9 +61,11 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
   const bool live = j < N;
   const int ch = h * N + (live ? j : 0);
 
-  extern __shared__ float lds[];
-  float* rk = lds;                   // [2][3][N]: r, k, decay of the current / next token
-  float* scratch = rk + 6 * N;       // 16
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  // [2][N] of (r, k, decay, bonus) by key channel for the current / next token: one 16-byte
+  // LDS read per channel in the sum below
+  float4* rk = reinterpret_cast<float4*>(lds);
+  float* scratch = lds + 8 * N;      // 16
   float* st = scratch + 16;          // [N][N] when NR == 0
   float sreg[NR > 0 ? NR : 1];
 
@@ -86,17 +88,11 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
     ng = ldf(gate + (int64_t)t0 * g_stride + ch);
   }
   const float my_nw = live ? norm_w[ch] : 0.f;
-  // the bonus by key channel, read by every thread: one more LDS row behind the state
-  float* ul = st + (NR > 0 ? 0 : N * N);
-  if (live) ul[j] = u[ch];
+  const float my_u = live ? u[ch] : 0.f;
 
   for (int a = 0; a < n; ++a) {
-    float* cur = rk + (a & 1) * 3 * N;
-    if (live) {
-      cur[j] = nr;
-      cur[N + j] = nk;
-      cur[2 * N + j] = nw;
-    }
+    const float4* cur = rk + (a & 1) * N;
+    if (live) rk[(a & 1) * N + j] = make_float4(nr, nk, nw, my_u);
     const float vj = nv, gj = ng;
     __syncthreads();
     if (a + 1 < n && live) {           // the next token's operands, in flight during the sums
@@ -112,16 +108,18 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
       if (NR > 0) {
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
-          const float kv = cur[N + i] * vj;
-          o += cur[i] * (sreg[i] + ul[i] * kv);
-          sreg[i] = cur[2 * N + i] * sreg[i] + kv;
+          const float4 c4 = cur[i];
+          const float kv = c4.y * vj;
+          o += c4.x * (sreg[i] + c4.w * kv);
+          sreg[i] = c4.z * sreg[i] + kv;
         }
       } else {
         for (int i = 0; i < N; ++i) {
+          const float4 c4 = cur[i];
           const float s = st[i * N + j];
-          const float kv = cur[N + i] * vj;
-          o += cur[i] * (s + ul[i] * kv);
-          st[i * N + j] = cur[2 * N + i] * s + kv;
+          const float kv = c4.y * vj;
+          o += c4.x * (s + c4.w * kv);
+          st[i * N + j] = c4.z * s + kv;
         }
       }
     }
@@ -165,7 +163,7 @@ static void launch_wkv_one(const void* r, const void* k, const void* v, const vo
                            const int32_t* row_back, const int32_t* row_fwd, const int32_t* pos,
                            void* out, int Trows, int H, int N, int slots, hipStream_t s) {
   const int threads = (N + 63) / 64 * 64;
-  const size_t lds = (size_t)(6 * N + 16 + (NR > 0 ? 0 : N * N) + N) * 4;
+  const size_t lds = (size_t)(8 * N + 16 + (NR > 0 ? 0 : N * N)) * 4;
   static bool attr = false;
   if (!attr) {          // dynamic LDS above 64 KB has to be allowed per kernel, once
     hipFuncSetAttribute(reinterpret_cast<const void*>(&wkv_recurrence_kernel<T, NR>),
