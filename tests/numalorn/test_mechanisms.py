@@ -361,7 +361,7 @@ def route_case(device, z, corr, r):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("r", [
-    {"experts": 8, "top": 4, "groups": {"count": 4, "keep": 3}},
+    {"experts": 10, "top": 4, "groups": {"count": 5, "keep": 3}},
     {"experts": 12, "top": 2, "groups": {"count": 3, "keep": 1}},
     {"experts": 6, "top": 3, "groups": {"count": 6, "keep": 4}},        # groups of one expert
     {"experts": 5, "top": 1}, {"experts": 7, "top": 7}])
