@@ -163,12 +163,17 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(
       const s16x8 pb_hi = __builtin_bit_cast(s16x8, hb), pb_lo = __builtin_bit_cast(s16x8, lb);
       const int q4 = c >> 2, p4 = c & 3;
       const int r0 = 4 * g4 + q4, r1 = 16 + 4 * g4 + q4;
+      // the accumulators are rescaled only on pages that moved some column's running maximum
+      // (wave-uniform test; a factor of exactly 1 changes nothing)
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0ull) {
+#pragma unroll
+        for (int m = 0; m < VT; ++m) o[m] *= alpha;
+      }
 #pragma unroll
       for (int m = 0; m < VT; ++m) {
         const s16x4 a0 = ds_read_tr16(c_lds + r0 * RS + 16 * m + 4 * p4);
         const s16x4 a1 = ds_read_tr16(c_lds + r1 * RS + 16 * m + 4 * p4);
         const s16x8 a = (s16x8){a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-        o[m] *= alpha;
         o[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(pb_hi), o[m], 0, 0, 0);
         o[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(pb_lo), o[m], 0, 0, 0);
       }
