@@ -28,11 +28,6 @@ SIZES = [("1b-class", 2048, 16, 4, 8192), ("8b-class", 4096, 32, 8, 14336),
 # (name, hidden, q heads, kv heads of the sparse decoder, experts, choices, expert ff)
 MOE_SIZES = [("moe-2k", 2048, 16, 4, 8, 2, 4096), ("moe-4k", 4096, 32, 8, 8, 2, 14336)]
 LAYERS, VOCAB, CHUNK = 4, 32000, 2048
-# The whole-model Numalorn runs at MOE_SIZES end in an illegal memory access in their first
-# 4,096-row prefill step on the GPU, although every kernel of that step passes alone at these
-# sizes (tests/kernels/test_numalorn_scale_gpu.py) and the engine passes at 2048-wide layers
-# with steps of some hundred rows: the cause is not found, so these sizes stay switched off.
-NUMALORN_SIZES_OFF = ("moe-2k", "moe-4k")
 
 
 def _configs(name, d, H, G, F):
@@ -117,9 +112,6 @@ def run(args) -> dict:
         name = size[0]
         if only and name not in only:
             continue
-        if arch == "numalorn" and name in NUMALORN_SIZES_OFF:
-            raise RuntimeError(f"--arch-compare numalorn: size {name} is switched off (unexplained "
-                               "GPU memory fault in its first large prefill step)")
         row = {}
         models = [x for x in getattr(args, "arch_models", "").split(",") if x]
         for mcfg in (_configs(*size) if arch == "livisun" else _moe_configs(*size)):

@@ -146,7 +146,11 @@ class NumalornLM:
         HN = mx.heads * mx.dim
         mixes = ops.token_shift_mix(x, lw["mu"], st["prev"], rs, rb, rf, pos,
                                     torch.empty((5, T, x.shape[1]), dtype=dt, device=x.device))
-        rkvg = torch.bmm(mixes[:4], lw["rkvg"].transpose(1, 2))             # [4, T, H*N]
+        # r, k, v, gate: four plain products (one batched call over the four [d, d] weights
+        # returned garbage from the vendor library at 4,096 rows of 4096-wide layers)
+        rkvg = torch.empty((4, T, HN), dtype=dt, device=x.device)
+        for s in range(4):
+            torch.mm(mixes[s], lw["rkvg"][s].t(), out=rkvg[s])
         zw = ops.matmul_nt(torch.tanh(ops.matmul_nt(mixes[4], lw["w1"])), lw["w2"])
         y = ops.wkv_recurrence(rkvg[0], rkvg[1], rkvg[2], zw, lw["w0"], lw["u"], rkvg[3], lw["gn"],
                                self.cfg.rms_eps, st["wkv"], rs, rb, rf, pos,

@@ -151,3 +151,41 @@ def test_latent_attention_32_heads_2048_token_prompts():
                           torch.tensor([0]), torch.tensor([tail]), torch.tensor([lens[0]]), out_t,
                           torch.zeros(H), sink, 0)
     assert rel(out_d[lens[0] - tail:lens[0]], out_t) < 2e-2
+
+
+def test_vendor_products_4096_rows():
+    """The library products of a 4096-wide layer at 4,096 rows, as the model calls them
+    (plain, with fp32 output, the four recurrence projections into slices of one buffer,
+    narrow N or K): a sample of rows against fp32 on the CPU.  (torch.bmm over the four
+    [4096, 4096] weights returned garbage here, which is why the model does not batch them.)"""
+    g = torch.Generator(device=DEV).manual_seed(5)
+    T, d = 4096, 4096
+    rows = torch.arange(0, T, 513, device=DEV)
+
+    def rnd(*shape, std=1.0):
+        return (torch.randn(*shape, generator=g, device=DEV) * std).bfloat16()
+
+    def check(got, x, w, tol=2e-2):
+        want = x[rows].float().cpu() @ w.float().cpu().t()
+        assert rel(got[rows], want) < tol
+
+    h = rnd(T, d)
+    for n_out, k in ((2048, d), (d, d), (64, d), (8, d)):
+        w = rnd(n_out, k, std=k ** -0.5)
+        check(ops.matmul_nt(h, w), h, w)
+    w = rnd(8, d, std=d ** -0.5)
+    check(ops.matmul_nt(h, w, out_dtype=torch.float32), h, w, 1e-3)
+    cq, uq = rnd(T, 1536), rnd(d, 1536, std=1536 ** -0.5)
+    check(ops.matmul_nt(cq, uq), cq, uq)
+    t64, w2 = rnd(T, 64), rnd(d, 64, std=0.125)
+    check(ops.matmul_nt(torch.tanh(t64), w2), torch.tanh(t64), w2)
+    mixes, rkvg = rnd(5, T, d), rnd(4, d, d, std=d ** -0.5)
+    got = torch.empty(4, T, d, dtype=torch.bfloat16, device=DEV)
+    for b in range(4):
+        torch.mm(mixes[b], rkvg[b].t(), out=got[b])
+        check(got[b], mixes[b], rkvg[b])
+    head = rnd(32000, d, std=d ** -0.5)
+    x2 = rnd(2, d)
+    want = x2.float().cpu() @ head.float().cpu().t()
+    assert rel(ops.matmul_nt(x2, head, out_dtype=torch.float32), want) < 1e-3
+    torch.cuda.synchronize()
