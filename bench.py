@@ -370,17 +370,14 @@ def main():
             raise SystemExit("bench: --arch-compare livisun | numalorn runs on one GPU")
         from replisense_rfq_amd.benchmarks import arch_compare
 
-        if args.arch_compare == "numalorn" and not args.arch_sizes:
-            # per-kernel times at a served model's step sizes, and the whole model through the
-            # engine at the largest configuration that runs (arch_compare.NUMALORN_SIZES_OFF)
+        extra = {}
+        if args.arch_compare == "numalorn" and not args.arch_models:
+            # besides the whole models: per-kernel times at a served model's step sizes
             from replisense_rfq_amd.benchmarks import arch_kernels
 
-            print(json.dumps({"metric": "arch_compare", "arch": "numalorn", "dtype": "bf16",
-                              "data": "synthetic", "kernels": arch_kernels.run(args),
-                              "engine_small": arch_compare.run_small(args)}), flush=True)
-            return
+            extra["kernels"] = arch_kernels.run(args)
         print(json.dumps({"metric": "arch_compare", "arch": args.arch_compare, "dtype": "bf16",
-                          "data": "synthetic", **arch_compare.run(args)}), flush=True)
+                          "data": "synthetic", **arch_compare.run(args), **extra}), flush=True)
         return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(_self_launch(args))

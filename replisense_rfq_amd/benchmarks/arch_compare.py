@@ -138,31 +138,3 @@ def run(args) -> dict:
         out["sizes"][name] = row
     return out
 
-
-def run_small(args) -> dict:
-    """Numalorn through the engine at the largest configuration that is known to run: two
-    2048-wide layers (16 heads over a 512-wide latent, 32 recurrent heads, 8 experts of width
-    4096 on the grouped GEMMs), 4 sequences, prompts of 300 / 70 / 200 tokens in one step,
-    then decode graphs."""
-    from ..models.config import numalorn_layers
-    from ..models.numalorn import NumalornLM
-    from ..models.weights import init_numalorn_weights
-
-    d = 2048
-    mcfg = LayeredConfig("cmp-numalorn-small", architecture="Numalorn", vocab_size=2000, hidden=d,
-                         canon_taps=0, residual_mult=0.5, logit_softcap=30.0,
-                         layers=numalorn_layers(2, 16, 128, 128, 768, 512, 32, 4096, 8, 2, 2, 1, 0))
-    dev = torch.device("cuda", 0)
-    w = init_numalorn_weights(mcfg, dev, torch.bfloat16, args.seed, keep_full=False)
-    eng = LLMEngine(EngineConfig(model=mcfg.name, max_num_seqs=4, max_kv_blocks=64,
-                                 max_batched_tokens=2048, max_model_len=512,
-                                 use_graphs=not args.no_graphs, graph_buckets=(4,), grammar=False,
-                                 prefix_cache=False, warm_prefix=False, jump_forward=False,
-                                 tune_gemm=False), model=NumalornLM(mcfg, dev, weights=w))
-    g = torch.Generator().manual_seed(args.seed)
-    prompts = [torch.randint(2, 2000, (n,), generator=g).tolist() for n in (300, 70, 200)]
-    _measure(eng, prompts, 8)
-    p_tps, d_tps, steps = _measure(eng, prompts, 32)
-    return {"layers": 2, "width": d, "prompts": [300, 70, 200], "prefill_tok_s": round(p_tps),
-            "decode_tok_s": round(d_tps), "decode_steps": steps,
-            "graph_steps": eng.runner.stats["graph_steps"]}
