@@ -55,7 +55,8 @@ bool launch_attn_latent_mfma(const void*, int64_t, int64_t, const void*, const i
 void launch_wkv_recurrence(bool, const void*, const void*, const void*, const void*, const void*,
                            int64_t, int64_t, int64_t, int64_t, int64_t, const float*, const float*,
                            const float*, float, float*, const int32_t*, const int32_t*,
-                           const int32_t*, const int32_t*, void*, int, int, int, int, hipStream_t);
+                           const int32_t*, const int32_t*, const int32_t*, int, void*, int, int, int,
+                           int, hipStream_t);
 void launch_moe_route_grouped(const float*, const float*, int, int, int, int, int, int32_t*, float*,
                               hipStream_t);
 void launch_moe_pair_up(bool, const void*, int64_t, const int32_t*, const void*, void*, int, int,
@@ -366,7 +367,7 @@ void wkv_recurrence(const Tensor& r, const Tensor& k, const Tensor& v, const Ten
                     const Tensor& w0, const Tensor& u, const Tensor& gate, const Tensor& norm_w,
                     double eps, const Tensor& state, const Tensor& row_state,
                     const Tensor& row_back, const Tensor& row_fwd, const Tensor& pos,
-                    const Tensor& out) {
+                    const OptT& run_rows, const Tensor& out) {
   const bool f32 = act_f32(r, "wkv_recurrence r");
   TORCH_CHECK(u.dim() == 2, "wkv_recurrence: u [H, N]");
   const int H = (int)u.size(0), N = (int)u.size(1), T = (int)r.size(0);
@@ -384,7 +385,9 @@ void wkv_recurrence(const Tensor& r, const Tensor& k, const Tensor& v, const Ten
       k.stride(0), v.stride(0), zw.stride(0), gate.stride(0), f32p(w0, "w0", HN), f32p(u, "u", HN),
       f32p(norm_w, "norm_w", HN), (float)eps, const_cast<float*>(f32p(state, "state")),
       i32p(row_state, "row_state", T), i32p(row_back, "row_back", T), i32p(row_fwd, "row_fwd", T),
-      i32p(pos, "positions", T), out.data_ptr(), T, H, N, (int)state.size(0) / 2, stream());
+      i32p(pos, "positions", T), run_rows.has_value() ? i32p(*run_rows, "run_rows", 0) : nullptr,
+      run_rows.has_value() ? (int)run_rows->numel() : 0, out.data_ptr(), T, H, N,
+      (int)state.size(0) / 2, stream());
 }
 
 // Latent attention on MFMA tiles: q [T, H, R] bf16 (the queries carried into the latent space;
@@ -493,7 +496,7 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("silu_mul_any(Tensor gate_up, Tensor(a!) out) -> ()");
   m.def("softcap(Tensor(a!) x, float cap) -> ()");
   m.def("token_shift_mix(Tensor x, Tensor mu, Tensor(a!) prev, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor(b!) out) -> ()");
-  m.def("wkv_recurrence(Tensor r, Tensor k, Tensor v, Tensor zw, Tensor w0, Tensor u, Tensor gate, Tensor norm_w, float eps, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor(b!) out) -> ()");
+  m.def("wkv_recurrence(Tensor r, Tensor k, Tensor v, Tensor zw, Tensor w0, Tensor u, Tensor gate, Tensor norm_w, float eps, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor? run_rows, Tensor(b!) out) -> ()");
   m.def("moe_route_grouped(Tensor z, Tensor correction, int top, int groups, int keep, Tensor(a!) ids, Tensor(b!) weights) -> ()");
   m.def("moe_pair_up(Tensor h, Tensor ids, Tensor w13, Tensor(a!) act) -> ()");
   m.def("moe_pair_down(Tensor act, Tensor ids, Tensor weights, Tensor w2, Tensor? base, Tensor(a!) out) -> ()");

@@ -52,9 +52,13 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
     const float* __restrict__ u, const float* __restrict__ norm_w, float eps,
     float* __restrict__ state, const int32_t* __restrict__ row_state,
     const int32_t* __restrict__ row_back, const int32_t* __restrict__ row_fwd,
-    const int32_t* __restrict__ pos, T* __restrict__ out, int H, int N, int slots) {
-  const int t0 = blockIdx.x, h = blockIdx.y;
-  if (row_back[t0] != 0) return;
+    const int32_t* __restrict__ pos, const int32_t* __restrict__ run_rows, T* __restrict__ out,
+    int H, int N, int slots) {
+  // with a list of the runs' first rows the grid holds only workgroups that work (-1: no run);
+  // without one, a workgroup per row, of which the runs' first rows work
+  const int t0 = run_rows != nullptr ? run_rows[blockIdx.x] : (int)blockIdx.x;
+  const int h = blockIdx.y;
+  if (t0 < 0 || row_back[t0] != 0) return;
   const int n = row_fwd[t0] + 1;
   const int code = row_state[t0];
   const int j = threadIdx.x;
@@ -161,7 +165,8 @@ static void launch_wkv_one(const void* r, const void* k, const void* v, const vo
                            int64_t gs, const float* w0, const float* u, const float* norm_w,
                            float eps, float* state, const int32_t* row_state,
                            const int32_t* row_back, const int32_t* row_fwd, const int32_t* pos,
-                           void* out, int Trows, int H, int N, int slots, hipStream_t s) {
+                           const int32_t* run_rows, int runs, void* out, int Trows, int H, int N,
+                           int slots, hipStream_t s) {
   const int threads = (N + 63) / 64 * 64;
   const size_t lds = (size_t)(8 * N + 16 + (NR > 0 ? 0 : N * N)) * 4;
   static bool attr = false;
@@ -170,10 +175,10 @@ static void launch_wkv_one(const void* r, const void* k, const void* v, const vo
                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     attr = true;
   }
-  hipLaunchKernelGGL((wkv_recurrence_kernel<T, NR>), dim3(Trows, H), dim3(threads), lds, s,
-                     (const T*)r, (const T*)k, (const T*)v, (const T*)zw, (const T*)gate, rs, ks,
-                     vs, zs, gs, w0, u, norm_w, eps, state, row_state, row_back, row_fwd, pos,
-                     (T*)out, H, N, slots);
+  hipLaunchKernelGGL((wkv_recurrence_kernel<T, NR>), dim3(run_rows != nullptr ? runs : Trows, H),
+                     dim3(threads), lds, s, (const T*)r, (const T*)k, (const T*)v, (const T*)zw,
+                     (const T*)gate, rs, ks, vs, zs, gs, w0, u, norm_w, eps, state, row_state,
+                     row_back, row_fwd, pos, run_rows, (T*)out, H, N, slots);
 }
 
 // Whether the head size fits (threads <= 256; the state matrix of a head in LDS).
@@ -184,11 +189,13 @@ void launch_wkv_recurrence(bool f32, const void* r, const void* k, const void* v
                            int64_t gs, const float* w0, const float* u, const float* norm_w,
                            float eps, float* state, const int32_t* row_state,
                            const int32_t* row_back, const int32_t* row_fwd, const int32_t* pos,
-                           void* out, int Trows, int H, int N, int slots, hipStream_t s) {
-  if (Trows == 0) return;
+                           const int32_t* run_rows, int runs, void* out, int Trows, int H, int N,
+                           int slots, hipStream_t s) {
+  if (Trows == 0 || (run_rows != nullptr && runs == 0)) return;
 #define WKV_GO(TT, NRR)                                                                         \
   launch_wkv_one<TT, NRR>(r, k, v, zw, gate, rs, ks, vs, zs, gs, w0, u, norm_w, eps, state,     \
-                          row_state, row_back, row_fwd, pos, out, Trows, H, N, slots, s)
+                          row_state, row_back, row_fwd, pos, run_rows, runs, out, Trows, H, N,  \
+                          slots, s)
   if (f32) {
     if (N == 64) WKV_GO(float, 64); else WKV_GO(float, 0);
   } else {

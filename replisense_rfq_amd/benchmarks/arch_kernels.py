@@ -76,8 +76,9 @@ def _wkv(T, H, N, rows, out, decode):
     nw = torch.ones(H * N, device=DEV)
     st = torch.zeros(128, H, N, N, device=DEV)
     y = torch.empty(T, H * N, dtype=torch.bfloat16, device=DEV)
-    t = _time(lambda: ops.wkv_recurrence(r, k, v, zw, w0, u, gate, nw, 1e-5, st, *rows, y))
-    seqs = int((rows[1] == 0).sum())
+    run = torch.nonzero(rows[1] == 0)[:, 0].to(torch.int32)       # the runs' first rows
+    t = _time(lambda: ops.wkv_recurrence(r, k, v, zw, w0, u, gate, nw, 1e-5, st, *rows, y, run))
+    seqs = int(run.numel())
     nbytes = T * H * N * 12 + (2 if decode else 1) * seqs * H * N * N * 4
     out["wkv_recurrence"] = _entry(t, nbytes, 6.0 * T * H * N * N)
 

@@ -93,6 +93,20 @@ class NumalornLM:
                              torch.zeros(size, dtype=torch.int32, device=self.device))
         return self._seq_ids[0][:n], self._seq_ids[1][:n]
 
+    def _run_rows(self, m):
+        """First row of every scheduled run of the step (decode section, then prefill section;
+        -1 for a sequence without rows: padding of a graph step), for the recurrence's grid."""
+        if self.device.type != "cuda" or not any(ly.mixer.kind == "wkv" for ly in self.cfg.layers):
+            return None
+        parts = []
+        if m.dec_q_len is not None and m.dec_q_len.numel():
+            parts.append(torch.where(m.dec_q_len > 0, m.dec_q_start, -1))
+        if m.pf_q_len is not None and m.pf_q_len.numel():
+            parts.append(torch.where(m.pf_q_len > 0, m.pf_q_start + m.num_decode, -1))
+        if not parts:
+            return None
+        return (parts[0] if len(parts) == 1 else torch.cat(parts)).to(torch.int32)
+
     def weight_bytes(self) -> int:
         tot = sum(v.numel() * v.element_size() for v in self.w.values() if isinstance(v, torch.Tensor))
         for lw in self.w["layers"]:
@@ -141,7 +155,7 @@ class NumalornLM:
 
     def _wkv(self, li, mx, lw, x, m, rows):
         T, dt = m.num_tokens, self.dtype
-        rs, rb, rf, pos = rows
+        rs, rb, rf, pos, runs = rows
         st = self.layer_state[li]
         HN = mx.heads * mx.dim
         mixes = ops.token_shift_mix(x, lw["mu"], st["prev"], rs, rb, rf, pos,
@@ -154,7 +168,7 @@ class NumalornLM:
         zw = ops.matmul_nt(torch.tanh(ops.matmul_nt(mixes[4], lw["w1"])), lw["w2"])
         y = ops.wkv_recurrence(rkvg[0], rkvg[1], rkvg[2], zw, lw["w0"], lw["u"], rkvg[3], lw["gn"],
                                self.cfg.rms_eps, st["wkv"], rs, rb, rf, pos,
-                               torch.empty((T, HN), dtype=dt, device=x.device))
+                               torch.empty((T, HN), dtype=dt, device=x.device), runs)
         return ops.matmul_nt(y, lw["o"])
 
     def _moe_buffers(self, T: int, f, d: int) -> MoEBuffers:
@@ -191,7 +205,8 @@ class NumalornLM:
         cfg, w = self.cfg, self.w
         T, eps, mult, dt = m.num_tokens, cfg.rms_eps, cfg.residual_mult, self.dtype
         pos = m.positions[:T]
-        rows = (m.extra["row_state"], m.extra["row_back"], m.extra["row_fwd"], pos)
+        rows = (m.extra["row_state"], m.extra["row_back"], m.extra["row_fwd"], pos,
+                self._run_rows(m))
         x = ops.embed_rows(m.input_ids[:T], w["embed"])
         h = x if dt == torch.float32 else x.to(dt)
         hbuf = None if dt == torch.float32 else h

@@ -1228,10 +1228,14 @@ def token_shift_mix(x, mu, prev, row_state, row_back, row_fwd, positions, out):
 
 
 def wkv_recurrence(r, k, v, zw, w0, u, gate, norm_w, eps: float, state, row_state, row_back,
-                   row_fwd, positions, out):
+                   row_fwd, positions, out, run_rows=None):
+    """``run_rows`` (int32, optional): the first row of every run of the step (-1: none).  The
+    kernel then launches one workgroup per (run, head) instead of one per (row, head) of which
+    most leave at once: with thousands of rows the few long-running ones otherwise end up
+    several to a SIMD."""
     if _gpu(r):
         _native.mix_ops().wkv_recurrence(r, k, v, zw, w0, u, gate, norm_w, float(eps), state,
-                                         row_state, row_back, row_fwd, positions, out)
+                                         row_state, row_back, row_fwd, positions, run_rows, out)
     else:
         ref.wkv_recurrence(r, k, v, zw, w0, u, gate, norm_w, eps, state, row_state, row_back,
                            row_fwd, positions, out)

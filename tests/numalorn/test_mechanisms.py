@@ -149,6 +149,40 @@ def test_wkv_recurrence_in_portions(device, H, N, cuts):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_wkv_runs_of_several_sequences_from_a_run_list(device):
+    """Three runs in one launch (one continues from its slot, two start), launched from the
+    list of their first rows with an empty entry in it: each as if it ran alone."""
+    g = torch.Generator().manual_seed(6)
+    H, N, eps = 3, 64, 1e-5
+    lens, slots, first = [37, 1, 70], [2, 0, 1], [5, 0, 0]
+    T = sum(lens)
+    r, k, v, gate, zw = (torch.randn(T, H * N, generator=g) * 0.5 for _ in range(5))
+    w0, u, nw = torch.randn(H * N, generator=g) - 1.5, torch.randn(H, N, generator=g), torch.randn(H * N, generator=g)
+    state = torch.randn(6, H, N, N, generator=g)
+    rs, rb, rf, pos = [], [], [], []
+    for n, s_, p0 in zip(lens, slots, first):
+        rs += [2 * s_] * n
+        rb += list(range(n))
+        rf += list(range(n - 1, -1, -1))
+        pos += list(range(p0, p0 + n))
+    st = state.clone().to(device)
+    out = torch.empty(T, H * N, device=device)
+    runs = i32([0, -1, 37, 38], device)
+    ops.wkv_recurrence(*(a.to(device) for a in (r, k, v, zw)), w0.to(device), u.to(device), gate.to(device),
+                       nw.to(device), eps, st, *(i32(x, device) for x in (rs, rb, rf, pos)), out, runs)
+    w = oracle.decay(zw.double(), w0.double()).view(T, H, N)
+    at = 0
+    for n, s_, p0 in zip(lens, slots, first):
+        sl = slice(at, at + n)
+        S0 = state[s_].double() if p0 > 0 else None       # half 0 of the slot
+        o, S1 = oracle.wkv_scan(*(a[sl].double().view(n, H, N) for a in (r, k, v)), w[sl], u.double(), S0)
+        want = oracle.rms_unit(o, eps).reshape(n, H * N) * nw.double() * oracle.silu(gate[sl].double())
+        close(out[sl], want, 1e-4)
+        close(st[3 + s_], S1, 1e-4)                        # other half
+        at += n
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_wkv_state_carried_far_and_bonus_only_now(device):
     """With decay ~ 1 on one channel a key from 300 tokens back still answers a matching
     query; with u = 0 the current token's own pair does not answer at all."""
